@@ -16,6 +16,10 @@ from .sogenex import SogenexConfig, sogenex_model_spec
 
 register_architecture("Sogenex", SogenexConfig.from_dict, sogenex_model_spec, aliases=("sogenex",))
 
-__all__ = ["TovasunConfig", "tovasun_model_spec", "SogenexConfig", "sogenex_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
+from .nusuvik import NusuvikConfig, nusuvik_model_spec
+
+register_architecture("Nusuvik", NusuvikConfig.from_dict, nusuvik_model_spec, aliases=("nusuvik",))
+
+__all__ = ["NusuvikConfig", "nusuvik_model_spec", "TovasunConfig", "tovasun_model_spec", "SogenexConfig", "sogenex_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
            "load_config", "lookup", "read_config_json", "register_architecture",
            "registered_architectures", "ConfigError", "Qwen2Config", "qwen2_model_spec"]

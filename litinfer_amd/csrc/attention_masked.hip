@@ -1063,14 +1063,15 @@ extern "C" int li_masked_attention_single(const float* q, int q_token_stride, in
 // ------------------------------------------------------------------------------------------- per-head products
 // out[t, h, j] = sum_k m[h, j, k] * x[t, h, k]: every head has a matrix of its own, [n_out, n_in], stored one after
 // the other.  x and out are addressed by a token stride and a head stride, so that a head's columns may lie inside
-// a wider row.  A block takes one head, HL_TOK tokens and 256 outputs: the tokens' inputs lie in LDS as float32, a
+// a wider row.  With `gate`, head h's outputs of token t are multiplied by sigmoid(gate[t * gate_stride + h]).
+// A block takes one head, HL_TOK tokens and 256 outputs: the tokens' inputs lie in LDS as float32, a
 // thread owns an output and reads its matrix row once for all the tokens.  Sums are float32, in the order of k.
 #define HL_TOK 8
 
 template <typename TX, typename TM, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(
     const TX* __restrict__ x, long x_token_stride, int x_head_stride, const TM* __restrict__ m, TO* __restrict__ out,
-    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in) {
+    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride) {
     extern __shared__ float xs[];                    // [HL_TOK][n_in]
     const int h = blockIdx.y, t0 = blockIdx.x * HL_TOK;
     const int nt = (T_ - t0 < HL_TOK) ? T_ - t0 : HL_TOK;
@@ -1117,8 +1118,10 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
             acc[tt] += __shfl_xor(acc[tt], 2, LI_WAVE);
         }
         if (on && part == 0)
-            for (int tt = 0; tt < nt; ++tt)
-                store_from_float(out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + j, acc[tt]);
+            for (int tt = 0; tt < nt; ++tt) {
+                const float f = gate ? 1.0f / (1.0f + expf(-gate[(size_t)(t0 + tt) * gate_stride + h])) : 1.0f;
+                store_from_float(out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + j, acc[tt] * f);
+            }
     }
 }
 
@@ -1129,7 +1132,7 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
 template <typename TX, typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
     const TX* __restrict__ x, long x_token_stride, int x_head_stride, const bf16_t* __restrict__ m, TO* __restrict__ out,
-    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in) {
+    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h2 = lane >> 5;
     const int head = blockIdx.y, t0 = blockIdx.x * 32;
     const int j0 = (blockIdx.z * 4 + w) * 32;
@@ -1154,6 +1157,11 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
     }
     if (t0 + ql >= T_) return;
+    if (gate) {
+        const float f = 1.0f / (1.0f + expf(-gate[(size_t)(t0 + ql) * gate_stride + head]));
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] *= f;
+    }
     TO* orow = out + (size_t)(t0 + ql) * o_token_stride + (size_t)head * o_head_stride + j0;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
@@ -1170,28 +1178,28 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
 
 template <typename TX, typename TO>
 static bool headwise_mfma(const void* x, long xts, int xhs, const void* m, void* out, long ots, int ohs, int T_, int nh,
-                          int n_out, int n_in, hipStream_t stream) {
+                          int n_out, int n_in, const float* gate, long gate_stride, hipStream_t stream) {
     const int ex = 16 / (int)sizeof(TX) / 2 * 2, eo = 4;       // elements that the 16-byte (32-byte) loads and the stores must start on
     if (T_ < 16 || n_in % 16 || n_out % 32 || xts % ex || xhs % ex || ots % eo || ohs % eo ||
         (uintptr_t)x % 16 || (uintptr_t)m % 16 || (uintptr_t)out % 16)
         return false;
     const dim3 grid((T_ + 31) / 32, nh, (n_out + 127) / 128);
     headwise_linear_mfma_kernel<TX, TO><<<grid, 256, 0, stream>>>((const TX*)x, xts, xhs, (const bf16_t*)m, (TO*)out, ots, ohs,
-                                                                  T_, n_out, n_in);
+                                                                  T_, n_out, n_in, gate, gate_stride);
     return true;
 }
 
 extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_stride, int x_head_stride, const void* m, int m_dtype,
                                   void* out, int out_dtype, long o_token_stride, int o_head_stride, int T_, int nh, int n_out,
-                                  int n_in, hipStream_t stream) {
-    if (T_ <= 0 || nh <= 0 || nh > 65535 || n_out <= 0 || n_in <= 0 || n_in > 2048) return LI_ERR_SIZE;
+                                  int n_in, const float* gate, long gate_stride, hipStream_t stream) {
+    if (T_ <= 0 || nh <= 0 || nh > 65535 || n_out <= 0 || n_in <= 0 || n_in > 2048 || (gate && gate_stride < nh)) return LI_ERR_SIZE;
     // many tokens against bfloat16 matrices of even sizes: the matrix cores
     if (m_dtype == LI_BF16) {
         bool took = false;
-        if (x_dtype == LI_F32 && out_dtype == LI_F32) took = headwise_mfma<float, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
-        else if (x_dtype == LI_F32 && out_dtype == LI_BF16) took = headwise_mfma<float, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
-        else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) took = headwise_mfma<bf16_t, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
-        else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
+        if (x_dtype == LI_F32 && out_dtype == LI_F32) took = headwise_mfma<float, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
+        else if (x_dtype == LI_F32 && out_dtype == LI_BF16) took = headwise_mfma<float, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) took = headwise_mfma<bf16_t, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
         if (took) return li_launch_status();
     }
     const int zs = (n_out + 63) / 64;
@@ -1202,10 +1210,10 @@ extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_strid
         constexpr int E = 16 / sizeof(TM);                                                                                 \
         if (n_in % E == 0 && ((uintptr_t)m % 16) == 0)                                                                     \
             headwise_linear_kernel<TX, TM, TO, true><<<grid, 256, lds, stream>>>(                                          \
-                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in); \
+                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride); \
         else                                                                                                               \
             headwise_linear_kernel<TX, TM, TO, false><<<grid, 256, lds, stream>>>(                                         \
-                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in); \
+                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride); \
         return li_launch_status();                                                                                         \
     }
     if (x_dtype == LI_F32 && m_dtype == LI_F32 && out_dtype == LI_F32) HL_GO(float, float, float)

@@ -657,59 +657,82 @@ extern "C" int li_qk_norm_pairs_store(float* qkv, int row_stride, int nh, int nk
     return li_launch_status();
 }
 
-// The same step for attention over a compressed cache.  A row of `qd` (float32) is [q | down]: q holds nh heads of
-// (dn + dr) columns, the last dr of each rotated; down holds `rank` latent columns and dr columns of one rotated key
-// part that all heads share.  The latent is RMS-normed (weights wc) and written to columns 0..rank-1 of the token's
-// page row, the rotated shared part behind it; the rotated part of every query head goes to columns rank.. of
-// that head's row in `qfull` (float32 rows of nh x (rank + dr): the first `rank` columns are filled by the product
-// with the keys' expansion matrix afterwards).
-template <typename T, int NT>
+// The same step for attention over a compressed cache.  `q` (float32 rows, may be absent: nh = 0) holds nh heads of
+// (dn + dr) columns, the last dr of each rotated; `down` (float32 rows, which may lie inside the same buffer) holds
+// `rank` latent columns and dr columns of one rotated key part that all heads share.  The latent is RMS-normed
+// (weights wc) and written to columns 0..rank-1 of the token's page row, the rotated shared part behind it; the
+// rotated part of every query head goes to columns rank.. of that head's row in `qfull` (float32 rows of
+// nh x (rank + dr): the first `rank` columns are filled by the product with the keys' expansion matrix afterwards).
+// `split`: 0 pairs neighbouring columns (2i, 2i + 1), 1 pairs column i with column i + dr/2.
+// Where the queries go through a latent of their own, `ql` holds its q_rank columns before the norm and `cq` takes
+// the RMS norm with weights wq (in the dtype of the product that follows).
+template <typename T, typename TQ, int NT>
 __global__ __launch_bounds__(NT) void latent_norm_pairs_store_kernel(
-    const float* __restrict__ qd, int row_stride, int nh, int dn, int dr, int rank, const float* __restrict__ wc, float eps,
-    const float* __restrict__ cosv, const float* __restrict__ sinv, const int* __restrict__ slot_map,
-    T* __restrict__ cache, float* __restrict__ qfull, int store) {
+    const float* __restrict__ q, long q_stride, int nh, int dn, int dr, const float* __restrict__ down, long down_stride,
+    int rank, const float* __restrict__ wc, float eps, const float* __restrict__ cosv, const float* __restrict__ sinv,
+    const int* __restrict__ slot_map, T* __restrict__ cache, float* __restrict__ qfull, int store, int split,
+    const float* __restrict__ ql, long ql_stride, int q_rank, const float* __restrict__ wq, TQ* __restrict__ cq) {
     __shared__ float red[NT / LI_WAVE];
     const int t = blockIdx.x, half = dr / 2;
-    const float* q = qd + (size_t)t * row_stride;
-    const float* down = q + (size_t)nh * (dn + dr);
+    const int second = split ? half : 1, step = split ? 1 : 2;       // a pair is (step * i, step * i + second)
     const float* c = cosv + (size_t)t * half;
     const float* sn = sinv + (size_t)t * half;
-    float* qf = qfull + (size_t)t * nh * (rank + dr);
-    for (int u = threadIdx.x; u < nh * half; u += NT) {
-        const int h = u / half, i = u % half;
-        const float* src = q + (size_t)h * (dn + dr) + dn + 2 * i;
-        float ra, rb;
-        rotate_pair(src[0], src[1], c[i], sn[i], ra, rb);
-        float* dst = qf + (size_t)h * (rank + dr) + rank + 2 * i;
-        dst[0] = ra; dst[1] = rb;
+    if (nh > 0) {
+        const float* qr = q + (size_t)t * q_stride;
+        float* qf = qfull + (size_t)t * nh * (rank + dr);
+        for (int u = threadIdx.x; u < nh * half; u += NT) {
+            const int h = u / half, i = u % half;
+            const float* src = qr + (size_t)h * (dn + dr) + dn + step * i;
+            float ra, rb;
+            rotate_pair(src[0], src[second], c[i], sn[i], ra, rb);
+            float* dst = qf + (size_t)h * (rank + dr) + rank + step * i;
+            dst[0] = ra; dst[second] = rb;
+        }
+    }
+    if (q_rank > 0) {
+        const float* lr = ql + (size_t)t * ql_stride;
+        float s = 0.f;
+        for (int j = threadIdx.x; j < q_rank; j += NT) s += lr[j] * lr[j];
+        s = block_sum<NT>(s, red);
+        const float inv = 1.0f / sqrtf(s / (float)q_rank + eps);
+        TQ* o = cq + (size_t)t * q_rank;
+        for (int j = threadIdx.x; j < q_rank; j += NT) store_from_float(o + j, wq[j] * lr[j] * inv);
     }
     if (!store) return;
+    const float* dw = down + (size_t)t * down_stride;
     float s = 0.f;
-    for (int j = threadIdx.x; j < rank; j += NT) s += down[j] * down[j];
+    for (int j = threadIdx.x; j < rank; j += NT) s += dw[j] * dw[j];
     s = block_sum<NT>(s, red);
     const float inv = 1.0f / sqrtf(s / (float)rank + eps);
     T* row = cache + (size_t)slot_map[t] * (rank + dr);
-    for (int j = threadIdx.x; j < rank; j += NT) store_from_float(row + j, down[j] * inv * wc[j]);
+    for (int j = threadIdx.x; j < rank; j += NT) store_from_float(row + j, dw[j] * inv * wc[j]);
     for (int i = threadIdx.x; i < half; i += NT) {
         float ra, rb;
-        rotate_pair(down[rank + 2 * i], down[rank + 2 * i + 1], c[i], sn[i], ra, rb);
-        store_from_float(row + rank + 2 * i, ra);
-        store_from_float(row + rank + 2 * i + 1, rb);
+        rotate_pair(dw[rank + step * i], dw[rank + step * i + second], c[i], sn[i], ra, rb);
+        store_from_float(row + rank + step * i, ra);
+        store_from_float(row + rank + step * i + second, rb);
     }
 }
 
-extern "C" int li_latent_norm_pairs_store(const float* qd, int row_stride, int nh, int dn, int dr, int rank, const float* wc,
-                                          float eps, const float* cosv, const float* sinv, const int* slot_map, void* cache,
-                                          int cache_dtype, float* qfull, int store, int T, hipStream_t stream) {
-    if (T <= 0 || nh <= 0 || dn < 0 || dr <= 0 || (dr & 1) || rank <= 0 || row_stride < nh * (dn + dr) + rank + dr)
+extern "C" int li_latent_norm_pairs_store(const float* q, long q_stride, int nh, int dn, int dr, const float* down,
+                                          long down_stride, int rank, const float* wc, float eps, const float* cosv,
+                                          const float* sinv, const int* slot_map, void* cache, int cache_dtype, float* qfull,
+                                          int store, int split, const float* ql, long ql_stride, int q_rank, const float* wq,
+                                          void* cq, int cq_dtype, int T, hipStream_t stream) {
+    if (T <= 0 || nh < 0 || dn < 0 || dr <= 0 || (dr & 1) || rank <= 0 || q_rank < 0) return LI_ERR_SIZE;
+    if ((nh > 0 && (!q || !qfull || q_stride < (long)nh * (dn + dr))) || (store && (!down || !cache || !slot_map || down_stride < rank + dr)) ||
+        (q_rank > 0 && (!ql || !wq || !cq || ql_stride < q_rank)))
         return LI_ERR_SIZE;
-    if (cache_dtype == LI_F32)
-        latent_norm_pairs_store_kernel<float, 256><<<T, 256, 0, stream>>>(qd, row_stride, nh, dn, dr, rank, wc, eps, cosv, sinv,
-                                                                          slot_map, (float*)cache, qfull, store);
-    else if (cache_dtype == LI_BF16)
-        latent_norm_pairs_store_kernel<bf16_t, 256><<<T, 256, 0, stream>>>(qd, row_stride, nh, dn, dr, rank, wc, eps, cosv, sinv,
-                                                                           slot_map, (bf16_t*)cache, qfull, store);
+#define LI_LN(T_, TQ_)                                                                                                          \
+    latent_norm_pairs_store_kernel<T_, TQ_, 256><<<T, 256, 0, stream>>>(q, q_stride, nh, dn, dr, down, down_stride, rank, wc, eps, \
+                                                                        cosv, sinv, slot_map, (T_*)cache, qfull, store, split, ql, \
+                                                                        ql_stride, q_rank, wq, (TQ_*)cq)
+    if (cache_dtype == LI_F32 && cq_dtype == LI_F32) LI_LN(float, float);
+    else if (cache_dtype == LI_BF16 && cq_dtype == LI_BF16) LI_LN(bf16_t, bf16_t);
+    else if (cache_dtype == LI_F32 && cq_dtype == LI_BF16) LI_LN(float, bf16_t);
+    else if (cache_dtype == LI_BF16 && cq_dtype == LI_F32) LI_LN(bf16_t, float);
     else return LI_ERR_DTYPE;
+#undef LI_LN
     return li_launch_status();
 }
 
@@ -819,5 +842,176 @@ extern "C" int li_diff_combine(const void* a1, const void* a2, int in_dtype, flo
     else if (in_dtype == LI_BF16 && out_dtype == LI_F32) DC(bf16_t, float);
     else return LI_ERR_DTYPE;
 #undef DC
+    return li_launch_status();
+}
+
+// ============================================================================================
+// A hashed pair-of-tokens embedding, layer norm with bias, the tanh form of GELU, two rows side by side.
+// ============================================================================================
+
+// out[t, :] = table[id(t), :] + pair[row(t), :] in float32.  row(t) is (prev * mul_prev + id * mul_cur) mod buckets
+// with prev the id of the token before t in its request, and row number `buckets` (the table's last) for a
+// request's first token (position 0) or where an id is no token of the vocabulary.  The token before a step's first
+// one of a request comes from `last[slot]`, which the same block then sets to the id of the request's last token of
+// this step: one block a segment touches a slot, and it reads before it writes.
+template <typename T>
+__global__ void pair_embedding_kernel(const int* __restrict__ ids, const int* __restrict__ id_src,
+                                      const int* __restrict__ feedback, const int* __restrict__ positions,
+                                      const int* __restrict__ seg_of_token, const int* __restrict__ q_start,
+                                      const int* __restrict__ q_len, const int* __restrict__ slots, int* __restrict__ last,
+                                      const T* __restrict__ table, const T* __restrict__ pair, float* __restrict__ out,
+                                      int H, int V, int buckets, long mul_prev, long mul_cur) {
+    const int t = blockIdx.x;
+    __shared__ int sid, sprev;
+    if (threadIdx.x == 0) {
+        auto id_of = [&](int u) {
+            int id = ids[u];
+            if (id_src) {
+                const int src = id_src[u];
+                if (src >= 0) id = feedback[src];
+            }
+            return id;
+        };
+        const int seg = seg_of_token[t], first = q_start[seg];
+        const int id = id_of(t);
+        int prev = -1;
+        if (positions[t] > 0) prev = (t > first) ? id_of(t - 1) : last[slots[seg]];
+        if (t == first) last[slots[seg]] = id_of(first + q_len[seg] - 1);
+        sid = id; sprev = prev;
+    }
+    __syncthreads();
+    const int id = sid, prev = sprev;
+    const bool ok = id >= 0 && id < V;
+    int row = buckets;
+    if (ok && prev >= 0 && prev < V) row = (int)(((long)prev * mul_prev + (long)id * mul_cur) % (long)buckets);
+    const T* e = table + (size_t)(ok ? id : 0) * H;
+    const T* p = pair + (size_t)row * H;
+    float* o = out + (size_t)t * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x)
+        o[j] = (ok ? load_as_float(e + j) : 0.f) + load_as_float(p + j);
+}
+
+extern "C" int li_pair_embedding(const int* ids, const int* id_src, const int* feedback, const int* positions,
+                                 const int* seg_of_token, const int* q_start, const int* q_len, const int* slots, int* last,
+                                 const void* table, const void* pair, int table_dtype, float* out, int T, int H, int V,
+                                 int buckets, long mul_prev, long mul_cur, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || V <= 0 || buckets <= 0 || mul_prev < 0 || mul_cur < 0 || (id_src && !feedback)) return LI_ERR_SIZE;
+    if (table_dtype == LI_F32)
+        pair_embedding_kernel<float><<<T, 256, 0, stream>>>(ids, id_src, feedback, positions, seg_of_token, q_start, q_len, slots,
+                                                            last, (const float*)table, (const float*)pair, out, H, V, buckets,
+                                                            mul_prev, mul_cur);
+    else if (table_dtype == LI_BF16)
+        pair_embedding_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, id_src, feedback, positions, seg_of_token, q_start, q_len, slots,
+                                                             last, (const bf16_t*)table, (const bf16_t*)pair, out, H, V, buckets,
+                                                             mul_prev, mul_cur);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b, one block a row; the row stays in registers (up to
+// PER elements a thread, longer rows are read again), mean and variance are two passes over it, all in float32.
+template <typename TO, int NT, int PER>
+__global__ __launch_bounds__(NT) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                        const float* __restrict__ b, float eps, TO* __restrict__ out, int H) {
+    __shared__ float red[NT / LI_WAVE];
+    const float* row = x + (size_t)blockIdx.x * H;
+    TO* o = out + (size_t)blockIdx.x * H;
+    float v[PER];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
+        v[i] = (j < H) ? row[j] : 0.f;
+        s += v[i];
+    }
+    for (int j = threadIdx.x + PER * NT; j < H; j += NT) s += row[j];
+    const float mean = block_sum<NT>(s, red) / (float)H;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
+        const float d = (j < H) ? v[i] - mean : 0.f;
+        ss += d * d;
+    }
+    for (int j = threadIdx.x + PER * NT; j < H; j += NT) { const float d = row[j] - mean; ss += d * d; }
+    ss = block_sum<NT>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
+        if (j < H) store_from_float(o + j, fmaf((v[i] - mean) * inv, w[j], b ? b[j] : 0.f));
+    }
+    for (int j = threadIdx.x + PER * NT; j < H; j += NT)
+        store_from_float(o + j, fmaf((row[j] - mean) * inv, w[j], b ? b[j] : 0.f));
+}
+
+extern "C" int li_layernorm(const float* x, const float* w, const float* b, float eps, void* out, int out_dtype, int T, int H,
+                            hipStream_t stream) {
+    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
+#define LI_LNORM(TO)                                                                                        \
+    {                                                                                                       \
+        if (T >= 256 || H <= 1024) layernorm_kernel<TO, 256, 16><<<T, 256, 0, stream>>>(x, w, b, eps, (TO*)out, H); \
+        else layernorm_kernel<TO, 1024, 8><<<T, 1024, 0, stream>>>(x, w, b, eps, (TO*)out, H);              \
+    }
+    if (out_dtype == LI_F32) LI_LNORM(float)
+    else if (out_dtype == LI_BF16) LI_LNORM(bf16_t)
+    else return LI_ERR_DTYPE;
+#undef LI_LNORM
+    return li_launch_status();
+}
+
+// out = gelu_tanh(x), element by element
+template <typename TI, typename TO>
+__global__ void gelu_tanh_kernel(const TI* __restrict__ x, TO* __restrict__ out, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) store_from_float(out + i, gelu_tanh(load_as_float(x + i)));
+}
+
+extern "C" int li_gelu_tanh(const void* x, int x_dtype, void* out, int out_dtype, long n, hipStream_t stream) {
+    if (n <= 0) return LI_ERR_SIZE;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (x_dtype == LI_F32 && out_dtype == LI_F32) gelu_tanh_kernel<float, float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, n);
+    else if (x_dtype == LI_F32 && out_dtype == LI_BF16) gelu_tanh_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>((const float*)x, (bf16_t*)out, n);
+    else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) gelu_tanh_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// out[t, :] = [a[t, :] | b[t, :]] for float32 rows a and b of H columns, in the dtype of out
+template <typename TO>
+__global__ void concat_rows_kernel(const float* __restrict__ a, const float* __restrict__ b, TO* __restrict__ out, int H) {
+    const int t = blockIdx.x;
+    TO* o = out + (size_t)t * 2 * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        store_from_float(o + j, a[(size_t)t * H + j]);
+        store_from_float(o + H + j, b[(size_t)t * H + j]);
+    }
+}
+
+extern "C" int li_concat_rows(const float* a, const float* b, void* out, int out_dtype, int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
+    if (out_dtype == LI_F32) concat_rows_kernel<float><<<T, 256, 0, stream>>>(a, b, (float*)out, H);
+    else if (out_dtype == LI_BF16) concat_rows_kernel<bf16_t><<<T, 256, 0, stream>>>(a, b, (bf16_t*)out, H);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// out[r, i] = silu(gu[r, i]) * gu[r, I + i] for float32 rows of gate and up values, in the dtype of out
+template <typename TO>
+__global__ void swiglu_rows_kernel(const float* __restrict__ gu, TO* __restrict__ out, long rows, int I) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * I) return;
+    const long r = idx / I;
+    const int i = (int)(idx % I);
+    const float g = gu[r * 2 * I + i], u = gu[r * 2 * I + I + i];
+    store_from_float(out + idx, u * (g / (1.0f + expf(-g))));
+}
+
+extern "C" int li_swiglu_rows(const float* gu, void* out, int out_dtype, long rows, int I, hipStream_t stream) {
+    if (rows <= 0 || I <= 0) return LI_ERR_SIZE;
+    const unsigned blocks = (unsigned)((rows * I + 255) / 256);
+    if (out_dtype == LI_F32) swiglu_rows_kernel<float><<<blocks, 256, 0, stream>>>(gu, (float*)out, rows, I);
+    else if (out_dtype == LI_BF16) swiglu_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gu, (bf16_t*)out, rows, I);
+    else return LI_ERR_DTYPE;
     return li_launch_status();
 }

@@ -13,6 +13,8 @@
 // ------------------------------------------------------------------------------------------------ router
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
 // largest (the lower index wins a tie), weights = softmax over the chosen logits.  gate[t] = sigmoid(wg . x).
+// mode 1: scores are sigmoid(logit), the choice goes by score + corr[e] inside the best groups of neighbouring
+// experts, the weights are the chosen scores over their sum.
 template <typename T> struct RouteVec;
 template <> struct RouteVec<float> { static constexpr int N = 4; };
 template <> struct RouteVec<bf16_t> { static constexpr int N = 8; };
@@ -38,10 +40,13 @@ template <typename TX, typename TW, int NT>
 __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x, long x_stride, const TW* __restrict__ wr,
                                                        const float* __restrict__ br, const TW* __restrict__ wg,
                                                        int* __restrict__ idx, float* __restrict__ wt, float* __restrict__ gate,
-                                                       int K, int E, int top, int vec) {
-    extern __shared__ __align__(16) float sm[];        // [K] the row, [E] the logits
+                                                       int K, int E, int top, int vec, int mode,
+                                                       const float* __restrict__ corr, int groups, int keep) {
+    extern __shared__ __align__(16) float sm[];        // [K] the row, [E] the logits, [E] the scores, [groups] the groups' scores
     float* xs = sm;
     float* lg = sm + ((K + 3) & ~3);
+    float* sc = lg + E;
+    float* gs = sc + E;
     const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const TX* row = x + (size_t)t * x_stride;
     for (int k = threadIdx.x; k < K; k += NT) xs[k] = load_as_float(row + k);
@@ -64,6 +69,46 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
     }
     __syncthreads();
     if (w != 0) return;
+    if (mode == 1) {
+        // scores s = sigmoid(logit); the choice goes by s + corr among the experts of the `keep` groups (of E / groups
+        // neighbours each) whose two largest choice values have the largest sum; the weights are the chosen s, normalised
+        for (int e = lane; e < E; e += 64) {
+            const float s = 1.0f / (1.0f + expf(-lg[e]));
+            sc[e] = s;
+            lg[e] = s + (corr ? corr[e] : 0.f);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (groups > 1 && keep < groups) {
+            const int per = E / groups;
+            for (int g = lane; g < groups; g += 64) {
+                float a = -INFINITY, b = -INFINITY;           // the largest and the second largest of the group
+                for (int e = g * per; e < (g + 1) * per; ++e) {
+                    const float v = lg[e];
+                    if (v > a) { b = a; a = v; } else if (v > b) b = v;
+                }
+                gs[g] = per > 1 ? a + b : a;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // a group is kept if fewer than `keep` groups come before it (a larger score, or an equal one and a lower number)
+            for (int g = lane; g < groups; g += 64) {
+                const float mine_s = gs[g];
+                int before = 0;
+                for (int o = 0; o < groups; ++o) {
+                    const float v = gs[o];
+                    before += (v > mine_s || (v == mine_s && o < g)) ? 1 : 0;
+                }
+                if (before >= keep)
+                    for (int e = g * per; e < (g + 1) * per; ++e) lg[e] = -INFINITY;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
     // wave 0 picks: `top` rounds of a maximum over the logits that are left
     float chosen = 0.f, mx = 0.f, sum = 0.f;
     int mine = -1;
@@ -81,7 +126,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
             if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
         }
         if (r == 0) mx = best;
-        const float ex = expf(best - mx);
+        const float ex = mode == 1 ? sc[bi] : expf(best - mx);
         sum += ex;
         if (lane == r) { mine = bi; chosen = ex; }
         if (lane == 0) lg[bi] = -INFINITY;
@@ -90,22 +135,26 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
+    if (mode == 1) sum += 1e-20f;
     if (lane < top) { idx[(size_t)t * top + lane] = mine; wt[(size_t)t * top + lane] = chosen / sum; }
 }
 
 extern "C" int li_moe_route(const void* x, int x_dtype, long x_stride, const void* wr, int w_dtype, const float* br, const void* wg,
-                            int* idx, float* wt, float* gate, int T, int K, int E, int top, hipStream_t stream) {
-    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (size_t)(K + E + 4) * 4 > 60000 || (wg && !gate))
+                            int* idx, float* wt, float* gate, int T, int K, int E, int top, int mode, const float* corr,
+                            int groups, int keep, hipStream_t stream) {
+    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (wg && !gate) || mode < 0 || mode > 1 ||
+        groups <= 0 || keep <= 0 || keep > groups || E % groups || (size_t)(K + 2 * E + groups + 4) * 4 > 60000)
         return LI_ERR_SIZE;
-    const size_t lds = (size_t)(((K + 3) & ~3) + E) * 4;
+    if (mode == 1 && (long)top > (long)keep * (E / groups)) return LI_ERR_SIZE;      // more choices than the kept groups hold
+    const size_t lds = (size_t)(((K + 3) & ~3) + 2 * E + groups) * 4;
     // whole 16-byte pieces of every matrix row (the gate row included)
     const int ve = w_dtype == LI_F32 ? 4 : 8;
     const int vec = K % ve == 0 && ((uintptr_t)wr % 16) == 0 && (!wg || ((uintptr_t)wg % 16) == 0);
     // few tokens: sixteen waves share a token's experts, so that a wave has one or two rows to go through
 #define MR(TX, TW)                                                                                                                \
     {                                                                                                                             \
-        if (T <= 128) moe_route_kernel<TX, TW, 1024><<<T, 1024, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec); \
-        else moe_route_kernel<TX, TW, 256><<<T, 256, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec);           \
+        if (T <= 128) moe_route_kernel<TX, TW, 1024><<<T, 1024, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec, mode, corr, groups, keep); \
+        else moe_route_kernel<TX, TW, 256><<<T, 256, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec, mode, corr, groups, keep);           \
     }
     if (x_dtype == LI_F32 && w_dtype == LI_F32) MR(float, float)
     else if (x_dtype == LI_BF16 && w_dtype == LI_BF16) MR(bf16_t, bf16_t)

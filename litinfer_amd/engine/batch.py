@@ -87,6 +87,7 @@ class StepContext:
         self.host_ctx_len: np.ndarray = None
         self.want_rows: torch.Tensor = None
         self.num_want = 0
+        self.embedding_out: torch.Tensor = None       # [T, H] float32: the embedding output, where the model keeps it
         self._slot_maps: List[torch.Tensor] = []
         self._attn: List[AttentionMeta] = []
         self._shared: Dict[Any, Any] = {}

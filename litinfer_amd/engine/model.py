@@ -74,8 +74,14 @@ class Model:
 
     # ---- cache ------------------------------------------------------------
     def cache_needs(self) -> Tuple[List[object], List[Optional[int]]]:
+        """What every entry of the execution order keeps, and, as one more entry behind them, what the
+        embedding keeps (per-request state of its own, if any): `cache.view(len(order))` is its view."""
         needs = [self.layers[e.layer].cache_need() for e in self.order]
         sources = [e.cache_from for e in self.order]
+        own = self.embedding.cache_need() if hasattr(self.embedding, "cache_need") else None
+        if own is not None:
+            needs.append(own)
+            sources.append(None)
         return needs, sources
 
     # ---- forward ----------------------------------------------------------
@@ -84,7 +90,14 @@ class Model:
         float32 logits [wanted, vocab] at the wanted rows (None if none)."""
         h = self.spec.hidden_size
         x = ctx.ws.buffer("model.residual", (ctx.num_tokens, h), torch.float32)
-        self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback, positions=ctx.positions)
+        own = hasattr(self.embedding, "cache_need") and self.embedding.cache_need() is not None
+        self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback, positions=ctx.positions, ctx=ctx,
+                               cache=cache.view(len(self.order)) if own else None)
+        ctx.embedding_out = None
+        if any(getattr(p, "keeps_embedding_output", False) for p in self.injections):
+            # an injection reads the embedding output again later: a copy beside the stream
+            ctx.embedding_out = ctx.ws.buffer("model.embedding_out", (ctx.num_tokens, h), torch.float32)
+            ops.cast(x, ctx.embedding_out)
         stream = ResidualStream(x, ctx.ws)
         stream.ws_dtype = self.rt.dtype
         for i, e in enumerate(self.order):

@@ -43,7 +43,12 @@ _SIGNATURES = {
         "li_rope_freq_table": [P, P, I, F, P, P, I],
         "li_rope_pairs_apply": [P, I, I, I, I, I, P, P, I],
         "li_qk_norm_pairs_store": [P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, I],
-        "li_latent_norm_pairs_store": [P, I, I, I, I, I, P, F, P, P, P, P, I, P, I, I],
+        "li_latent_norm_pairs_store": [P, L, I, I, I, P, L, I, P, F, P, P, P, P, I, P, I, I, P, L, I, P, P, I, I],
+        "li_pair_embedding": [P, P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, L, L],
+        "li_layernorm": [P, P, P, F, P, I, I, I],
+        "li_gelu_tanh": [P, I, P, I, L],
+        "li_concat_rows": [P, P, P, I, I, I],
+        "li_swiglu_rows": [P, P, I, L, I],
         "li_sinusoid_add": [P, P, P, I, I],
         "li_scale_softcap": [P, L, F, F],
         "li_paged_store": [P, L, I, I, I, P, I, I, I, P, I, I, I, P, I, P, I, I],
@@ -55,7 +60,7 @@ _SIGNATURES = {
         "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I],
     },
     "moe": {
-        "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I],
+        "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I, I, P, I, I],
         "li_moe_plan": [P, I, I, I, P, I, P, P, I],
         "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, I, I],
         "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I],
@@ -65,7 +70,7 @@ _SIGNATURES = {
         "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L, P, I, I],
-        "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
+        "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, P, L],
     },
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
@@ -473,29 +478,118 @@ def qk_norm_pairs_store(qkv: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, 
              0 if k is None else v.data_ptr(), _DT[k.dtype] if k is not None else 0, page_size, int(k is not None), t)
 
 
-def latent_norm_pairs_store(qd: torch.Tensor, nh: int, dn: int, dr: int, rank: int, wc: torch.Tensor, eps: float,
+def latent_norm_pairs_store(qd: Optional[torch.Tensor], nh: int, dn: int, dr: int, rank: int, wc: torch.Tensor, eps: float,
                             cos: torch.Tensor, sin: torch.Tensor, slot_map: Optional[torch.Tensor],
-                            cache: Optional[torch.Tensor], qfull: torch.Tensor) -> None:
-    """qd float32 rows [q (nh x (dn + dr)) | latent (rank) | shared rotated key part (dr)].  The latent is
-    RMS-normed and written with the rotated shared part to the token's page row [rank + dr]; every query head's
-    rotated part goes to columns rank.. of its row in qfull [T, nh, rank + dr] (float32)."""
-    _gpu(qd, wc, cos, sin, slot_map, cache, qfull)
-    t = qd.shape[0]
-    _chk(_rows_ok(qd) and qd.dtype is torch.float32 and qd.shape[1] >= nh * (dn + dr) + rank + dr,
-         "latent_norm_pairs_store: qd")
+                            cache: Optional[torch.Tensor], qfull: Optional[torch.Tensor], down: Optional[torch.Tensor] = None,
+                            half_split: bool = False, q_latent: Optional[torch.Tensor] = None,
+                            wq: Optional[torch.Tensor] = None, cq: Optional[torch.Tensor] = None) -> None:
+    """qd float32 rows [q (nh x (dn + dr)) | latent (rank) | shared rotated key part (dr)]; with `down` (float32 rows
+    [latent | shared part], which may be a view of columns inside a wider buffer) qd holds the queries alone, and may
+    be None: then no query is touched.  The latent is RMS-normed and written with the rotated shared part to the
+    token's page row [rank + dr]; every query head's rotated part goes to columns rank.. of its row in qfull
+    [T, nh, rank + dr] (float32).  Pairs are neighbouring columns, or column i with column i + dr/2 (`half_split`).
+    With `q_latent` (float32 rows, a view is fine) also cq = the RMS norm of those rows with weights wq."""
+    _gpu(qd, wc, cos, sin, slot_map, cache, qfull, down, q_latent, wq, cq)
+    t = cos.shape[0]
+    if qd is None:
+        nh = 0
+    if nh:
+        need = nh * (dn + dr) + (0 if down is not None else rank + dr)
+        _chk(_rows_ok(qd) and qd.dtype is torch.float32 and qd.shape[0] == t and qd.shape[1] >= need, "latent_norm_pairs_store: qd")
+        _chk(qfull is not None and qfull.shape == (t, nh, rank + dr) and qfull.is_contiguous() and qfull.dtype is torch.float32,
+             "latent_norm_pairs_store: qfull")
+    if down is None and nh:
+        down = qd[:, nh * (dn + dr):]
     _chk(dr % 2 == 0 and dr > 0, "latent_norm_pairs_store: the rotated size must be even")
     _check_tables("latent_norm_pairs_store", t, dr, cos, sin, slot_map if cache is not None else None)
     _chk(wc.dtype is torch.float32 and wc.numel() == rank and wc.is_contiguous(), "latent_norm_pairs_store: norm weight")
-    _chk(qfull.shape == (t, nh, rank + dr) and qfull.is_contiguous() and qfull.dtype is torch.float32,
-         "latent_norm_pairs_store: qfull")
     if cache is not None:
+        _chk(down is not None and _rows_ok(down) and down.dtype is torch.float32 and down.shape == (t, rank + dr),
+             "latent_norm_pairs_store: the rows of latent and shared key part")
         _chk(cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + dr and cache.is_contiguous()
              and cache.dtype in _DT and slot_map is not None, "latent_norm_pairs_store: cache [pages, 1, page, rank + dr]")
-    if t:
-        _run("elementwise", "li_latent_norm_pairs_store", qd.data_ptr(), qd.stride(0), nh, dn, dr, rank, wc.data_ptr(),
+    q_rank = 0
+    if q_latent is not None:
+        q_rank = q_latent.shape[1]
+        _chk(_rows_ok(q_latent) and q_latent.dtype is torch.float32 and q_latent.shape[0] == t and q_rank > 0
+             and wq is not None and wq.dtype is torch.float32 and wq.numel() == q_rank and wq.is_contiguous()
+             and cq is not None and cq.shape == (t, q_rank) and cq.is_contiguous() and cq.dtype in _DT,
+             "latent_norm_pairs_store: the queries' latent, its norm weight and its output")
+    if t and (nh or cache is not None or q_rank):
+        _run("elementwise", "li_latent_norm_pairs_store", qd.data_ptr() if nh else 0, qd.stride(0) if nh else 0, nh, dn, dr,
+             down.data_ptr() if cache is not None else 0, down.stride(0) if cache is not None else 0, rank, wc.data_ptr(),
              float(eps), cos.data_ptr(), sin.data_ptr(), 0 if cache is None else slot_map.data_ptr(),
-             0 if cache is None else cache.data_ptr(), _DT[cache.dtype] if cache is not None else 0, qfull.data_ptr(),
-             int(cache is not None), t)
+             0 if cache is None else cache.data_ptr(), _DT[cache.dtype] if cache is not None else 0,
+             qfull.data_ptr() if nh else 0, int(cache is not None), int(bool(half_split)),
+             q_latent.data_ptr() if q_rank else 0, q_latent.stride(0) if q_rank else 0, q_rank,
+             wq.data_ptr() if q_rank else 0, cq.data_ptr() if q_rank else 0, _DT[cq.dtype] if q_rank else 0, t)
+
+
+def pair_embedding(ids: torch.Tensor, table: torch.Tensor, pair: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
+                   seg_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+                   last: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int,
+                   id_src: Optional[torch.Tensor] = None, feedback: Optional[torch.Tensor] = None) -> None:
+    """out[t, :] = table[id(t), :] + pair[row(t), :] as float32, row(t) = (prev * mul_prev + id * mul_cur) mod buckets
+    with prev the id of the token before t in its request, and the last row (number `buckets`) for a request's first
+    token.  `last` [slots] int32 holds every live request's last token between steps and is brought up to date;
+    the other arrays are the step's (segment of a token, a segment's first token, its length, its slot)."""
+    _gpu(ids, table, pair, out, positions, seg_of_token, q_start, q_len, slots, last, id_src, feedback)
+    t, h = out.shape
+    nseg = q_start.numel()
+    _chk(out.dtype is torch.float32 and out.is_contiguous() and _ids_ok(ids, id_src, feedback, t), "pair_embedding: out, ids")
+    _chk(table.dim() == 2 and table.shape[1] == h and table.is_contiguous() and table.dtype in _DT
+         and pair.shape == (buckets + 1, h) and pair.is_contiguous() and pair.dtype is table.dtype and buckets > 0
+         and mul_prev >= 0 and mul_cur >= 0, "pair_embedding: the tables")
+    for a_, n_ in ((positions, t), (seg_of_token, t), (q_start, nseg), (q_len, nseg), (slots, nseg)):
+        _chk(a_.dtype is torch.int32 and a_.numel() == n_ and a_.is_contiguous(), "pair_embedding: the step's index arrays")
+    _chk(last.dtype is torch.int32 and last.is_contiguous() and last.dim() == 1, "pair_embedding: the last tokens")
+    if t:
+        _run("elementwise", "li_pair_embedding", ids.data_ptr(), 0 if id_src is None else id_src.data_ptr(),
+             0 if id_src is None else feedback.data_ptr(), positions.data_ptr(), seg_of_token.data_ptr(), q_start.data_ptr(),
+             q_len.data_ptr(), slots.data_ptr(), last.data_ptr(), table.data_ptr(), pair.data_ptr(), _DT[table.dtype],
+             out.data_ptr(), t, h, table.shape[0], int(buckets), int(mul_prev), int(mul_cur))
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float, out: torch.Tensor) -> None:
+    """out = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias, row by row, in float32."""
+    _gpu(x, weight, bias, out)
+    _chk(x.dim() == 2 and x.shape == out.shape and x.is_contiguous() and out.is_contiguous() and x.dtype is torch.float32
+         and out.dtype in _DT, "layernorm: x float32 and out must be contiguous [T, H] of one shape")
+    for w_ in (weight, bias):
+        _chk(w_ is None or (w_.dtype is torch.float32 and w_.numel() == x.shape[1] and w_.is_contiguous()),
+             "layernorm: weight and bias must be float32 [H]")
+    if x.shape[0]:
+        _run("elementwise", "li_layernorm", x.data_ptr(), weight.data_ptr(), 0 if bias is None else bias.data_ptr(), float(eps),
+             out.data_ptr(), _DT[out.dtype], x.shape[0], x.shape[1])
+
+
+def gelu_tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))."""
+    _gpu(x, out)
+    _chk(x.shape == out.shape and x.is_contiguous() and out.is_contiguous() and x.dtype in _DT and out.dtype in _DT
+         and (x.dtype is torch.float32 or out.dtype is x.dtype), "gelu_tanh: x, out")
+    if x.numel():
+        _run("elementwise", "li_gelu_tanh", x.data_ptr(), _DT[x.dtype], out.data_ptr(), _DT[out.dtype], x.numel())
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, :] = [a[t, :] | b[t, :]] for float32 a and b [T, H], in the dtype of out [T, 2H]."""
+    _gpu(a, b, out)
+    t, h = a.shape
+    _chk(a.dtype is torch.float32 and b.dtype is torch.float32 and b.shape == a.shape and a.is_contiguous() and b.is_contiguous()
+         and out.shape == (t, 2 * h) and out.is_contiguous() and out.dtype in _DT, "concat_rows: a, b [T, H] float32, out [T, 2H]")
+    if t:
+        _run("elementwise", "li_concat_rows", a.data_ptr(), b.data_ptr(), out.data_ptr(), _DT[out.dtype], t, h)
+
+
+def swiglu_rows(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r, i] = silu(gate_up[r, i]) * gate_up[r, I + i] for float32 gate_up [R, 2I]; out [R, I] in its own dtype."""
+    _gpu(gate_up, out)
+    r, inter = out.shape
+    _chk(gate_up.shape == (r, 2 * inter) and gate_up.is_contiguous() and out.is_contiguous()
+         and gate_up.dtype is torch.float32 and out.dtype in _DT, "swiglu_rows: gate_up float32 [R, 2I], out [R, I]")
+    if r:
+        _run("elementwise", "li_swiglu_rows", gate_up.data_ptr(), out.data_ptr(), _DT[out.dtype], r, inter)
 
 
 _CUS: Dict[int, int] = {}
@@ -660,11 +754,13 @@ def masked_tiles_take(dk: int, dv: int) -> bool:
 
 
 def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m: torch.Tensor, out: torch.Tensor,
-                    o_token_stride: int, o_head_stride: int, tokens: int) -> None:
+                    o_token_stride: int, o_head_stride: int, tokens: int, gate: Optional[torch.Tensor] = None) -> None:
     """out[t, h, j] = sum_k m[h, j, k] * x[t, h, k] for m [heads, n_out, n_in]; head h of token t starts at
-    t * token_stride + h * head_stride in x (n_in values) and in out (n_out values)."""
-    _gpu(x, m, out)
+    t * token_stride + h * head_stride in x (n_in values) and in out (n_out values).  With `gate` (float32 rows
+    [tokens, heads], a view of columns is fine) head h's outputs of token t are multiplied by sigmoid(gate[t, h])."""
+    _gpu(x, m, out, gate)
     nh, n_out, n_in = m.shape
+    _chk(gate is None or (_rows_ok(gate) and gate.dtype is torch.float32 and gate.shape == (tokens, nh)), "headwise_linear: gate")
     _chk(m.is_contiguous() and m.dtype in _DT and x.dtype in _DT and out.dtype in _DT and x.is_contiguous()
          and out.is_contiguous(), "headwise_linear: operands")
     _chk(x.numel() >= (tokens - 1) * x_token_stride + (nh - 1) * x_head_stride + n_in
@@ -675,7 +771,7 @@ def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m:
     if tokens:
         _run("attention_masked", "li_headwise_linear", x.data_ptr(), _DT[x.dtype], int(x_token_stride), int(x_head_stride),
              m.data_ptr(), _DT[m.dtype], out.data_ptr(), _DT[out.dtype], int(o_token_stride), int(o_head_stride),
-             tokens, nh, n_out, n_in)
+             tokens, nh, n_out, n_in, 0 if gate is None else gate.data_ptr(), 0 if gate is None else gate.stride(0))
 
 
 # ---------------------------------------------------------------------- gemm
@@ -1455,23 +1551,34 @@ def moe_max_tiles(tokens: int, top: int, experts: int, tile_rows: int = MOE_TILE
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], gate_row: Optional[torch.Tensor],
-              idx: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor]) -> None:
+              idx: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor], scores: str = "softmax_chosen",
+              correction: Optional[torch.Tensor] = None, groups: int = 1, keep_groups: int = 1) -> None:
     """idx [T, top] int32: the experts with the largest logits x router^T + bias (float32 sums; the lower index wins a
-    tie); wt [T, top] float32: softmax over the chosen logits; gate [T] = sigmoid(x . gate_row) where a row is given."""
-    _gpu(x, router, bias, gate_row, idx, wt, gate)
+    tie); wt [T, top] float32: softmax over the chosen logits; gate [T] = sigmoid(x . gate_row) where a row is given.
+    With scores = "sigmoid" an expert's score is sigmoid(logit); the choice goes by score + correction[e], and only
+    among the experts of the `keep_groups` groups (of experts / groups neighbours each) whose two largest choice
+    values have the largest sum; wt = the chosen scores over their sum (+ 1e-20)."""
+    _gpu(x, router, bias, gate_row, idx, wt, gate, correction)
     t, k = x.shape
     e, top = router.shape[0], idx.shape[1]
+    _chk(scores in ("softmax_chosen", "sigmoid"), "moe_route: scores")
+    mode = 1 if scores == "sigmoid" else 0
+    _chk(correction is None or (mode == 1 and correction.dtype is torch.float32 and correction.numel() == e
+                                and correction.is_contiguous()), "moe_route: correction")
+    _chk(1 <= keep_groups <= groups and e % groups == 0 and (mode == 1 or groups == 1)
+         and (mode == 0 or top <= keep_groups * (e // groups)), "moe_route: groups")
     _chk(x.dtype in _DT and _rows_ok(x) and router.dtype in _DT and router.is_contiguous() and router.shape == (e, k)
          and (bias is None or (bias.dtype is torch.float32 and bias.numel() == e and bias.is_contiguous())), "moe_route: x, router, bias")
     _chk(idx.dtype is torch.int32 and idx.is_contiguous() and idx.shape == (t, top) and wt.dtype is torch.float32 and wt.is_contiguous()
          and wt.shape == (t, top) and 1 <= top <= min(e, 64), "moe_route: idx, wt [T, top], top at most 64")
     _chk((gate_row is None) == (gate is None) and (gate_row is None or (gate_row.dtype is router.dtype and gate_row.numel() == k
          and gate_row.is_contiguous() and gate.dtype is torch.float32 and gate.numel() == t and gate.is_contiguous())), "moe_route: gate")
-    _chk((k + e) * 4 <= 60000, "moe_route: the row and the logits must fit 60 KB of LDS")
+    _chk((k + 2 * e + groups + 4) * 4 <= 60000, "moe_route: the row and the logits must fit 60 KB of LDS")
     if t:
         _run("moe", "li_moe_route", x.data_ptr(), _DT[x.dtype], x.stride(0), router.data_ptr(), _DT[router.dtype],
              0 if bias is None else bias.data_ptr(), 0 if gate_row is None else gate_row.data_ptr(), idx.data_ptr(), wt.data_ptr(),
-             0 if gate is None else gate.data_ptr(), t, k, e, top)
+             0 if gate is None else gate.data_ptr(), t, k, e, top, mode, 0 if correction is None else correction.data_ptr(),
+             int(groups), int(keep_groups))
 
 
 def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: torch.Tensor, pair_row: torch.Tensor,

@@ -123,5 +123,55 @@ class SandwichBlock(Block):
             self.token_input.forward(stream, ctx, after)
 
 
+class ParallelBlock(Block):
+    """One norm, two readers: with h = norm1(x), x += mixer(h) + ffn(h).  Both sublayers add into the stream through
+    their last product (32-bit adds); a layer may lack the feed-forward."""
+
+    def __init__(self, spec, rt, parts):
+        super().__init__(spec, rt)
+        self.norm1 = build_part("norm", parts["norm1"], rt)
+        self.mixer = build_part("mixer", parts["mixer"], rt)
+        self.ffn = build_part("feed_forward", parts["feed_forward"], rt) if parts.get("feed_forward") is not None else None
+        self._all = tuple(p for p in (self.norm1, self.mixer, self.ffn) if p is not None)
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._all)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def batch_needs(self):
+        needs = super().batch_needs()
+        for p in self._all:
+            needs = needs.merged(p.batch_needs())
+        return needs
+
+    def expected_params(self):
+        e = {}
+        for p in self._all:
+            e.update(p.expected_params())
+        return e
+
+    def load_params(self, get):
+        for p in self._all:
+            p.load_params(get)
+
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, stream, ctx, cache):
+        after = stream.next_norm                   # the norm that reads the stream after this block
+        stream.next_norm = None                    # (between the two sublayers nobody reads the sum)
+        # the normed rows must outlive the mixer: the feed-forward reads them too
+        h = stream.normed(self.norm1, ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype))
+        self.mixer.forward(h, stream, ctx, cache)
+        if self.ffn is not None:
+            stream.next_norm = after
+            self.ffn.forward(h, stream, ctx)
+        stream.next_norm = None
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich", SandwichBlock)

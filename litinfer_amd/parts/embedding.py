@@ -11,7 +11,8 @@ Options that other designs use: the embedding may add a sinusoidal position vect
 (`sinusoid_base` b: column 2i gets sin(p b^(-2i/H)), column 2i+1 the cosine of the same
 angle; the frequencies are worked out once in float64 and rounded to float32, the angle is
 float(p) * f in float32); the head may scale its logits (`logit_scale`) and cap them
-(`softcap` c: c * tanh(logits / c)), in that order."""
+(`softcap` c: c * tanh(logits / c)), in that order.  `PairHashEmbedding` adds a row of a second, hashed table
+that the token and its predecessor choose together."""
 from __future__ import annotations
 
 import torch
@@ -47,12 +48,56 @@ class TokenEmbedding(Part):
             i = torch.arange((self.hidden + 1) // 2, dtype=torch.float64)
             self.freq = self.rt.vector(torch.pow(torch.tensor(self.sinusoid_base, dtype=torch.float64), -2.0 * i / self.hidden))
 
-    def forward(self, ids, out, id_src=None, feedback=None, positions=None):
+    def cache_need(self):
+        """Per-request state that the embedding keeps (none here); see `Mixer.cache_need`."""
+        return None
+
+    def forward(self, ids, out, id_src=None, feedback=None, positions=None, ctx=None, cache=None):
         ops.embedding(ids, self.table, out, id_src, feedback)
         if self.freq is not None:
             if positions is None:
                 raise ValueError("embedding: the position vector needs the tokens' positions")
             ops.sinusoid_add(out, positions, self.freq)
+        return out
+
+
+class PairHashEmbedding(TokenEmbedding):
+    """The token's row plus a row of a second table that is chosen by the token AND the one before it in its
+    request: row (previous * mul_prev + token * mul_cur) mod buckets of `pair_param` [buckets + 1, hidden], and the
+    table's last row for a request's first token.  The token before a step's first one is per-request state: one
+    int32 a state slot, kept up to date by the kernel that gathers (so tokens chosen on the device count too)."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        a = spec.args
+        self.buckets, self.mul_prev, self.mul_cur = int(a["buckets"]), int(a["mul_prev"]), int(a["mul_cur"])
+        if self.buckets <= 0 or self.mul_prev < 0 or self.mul_cur < 0:
+            raise ValueError("pair embedding: buckets must be positive and the multipliers not negative")
+        if (self.vocab - 1) * (self.mul_prev + self.mul_cur) >= 1 << 62:
+            raise ValueError("pair embedding: the multipliers are too large for 64-bit sums")
+        self.pair_param = self.prefix + str(a.get("pair_param", "bigram"))
+        self.pair = None
+
+    def cache_need(self):
+        from .base import StateNeed
+        return StateNeed((1,), torch.int32, "last_token")
+
+    def expected_params(self):
+        return {**super().expected_params(), self.pair_param: ParamSpec((self.buckets + 1, self.hidden))}
+
+    def load_params(self, get):
+        super().load_params(get)
+        self.pair = self.rt.matrix(get(self.pair_param))
+        if self.pair.dtype is not self.table.dtype:
+            self.pair = self.pair.to(self.table.dtype)
+
+    def forward(self, ids, out, id_src=None, feedback=None, positions=None, ctx=None, cache=None):
+        if ctx is None or cache is None or cache.state is None:
+            raise ValueError("pair embedding: needs the step's segments and its state (the requests' last tokens)")
+        ops.pair_embedding(ids, self.table, self.pair, out, ctx.positions, ctx.seg_of_token, ctx.q_start, ctx.q_len,
+                           ctx.state_slots, cache.state.view(-1), self.buckets, self.mul_prev, self.mul_cur, id_src, feedback)
+        if self.freq is not None:
+            ops.sinusoid_add(out, ctx.positions, self.freq)
         return out
 
 
@@ -100,4 +145,5 @@ class LinearHead(Part):
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("embedding", "pair_hash_embedding", PairHashEmbedding)
 register_part("head", "linear_head", LinearHead)

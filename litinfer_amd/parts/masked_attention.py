@@ -17,6 +17,10 @@ never carried out per key: q_h . (Wuk_h c) = (Wuk_h^T q_h) . c, and sum_j p_j Wu
 Wuv_h (sum_j p_j c_j), so the attention runs over the cached rows themselves, one kv head of
 rank + rot_dim key columns whose first `rank` are also the value, with a per-head product before
 (queries into the latent space) and one after it (the summed latent into the head's value space).
+Options: the queries may go through a latent of their own (`q_rank` > 0: c_q = RMS norm of Wdq xn with weights
+`q_down_norm`, q = Wuq c_q); every head's output may be multiplied by a sigmoid gate of the mixer's input
+(`head_gate`: sigmoid(Wg xn)_h, one row of Wg a head); the position part says how it pairs columns (`layout`:
+neighbouring ones, or column i with column i + rot_dim/2).
 """
 from __future__ import annotations
 
@@ -116,20 +120,23 @@ class LatentAttention(Mixer):
         self.dr = int(a["rot_dim"])                  # rotated columns
         self.dv = int(a.get("value_dim") or self.dn)
         self.rank = int(a["kv_rank"])
+        self.q_rank = int(a.get("q_rank") or 0)      # 0: the queries are one product of the input
+        self.head_gate = bool(a.get("head_gate", False))
         self.window = int(a.get("window") or 0)
         self.keep_first = int(a.get("keep_first") or 0) if self.window else 0
         self.softcap = float(a.get("softcap") or 0.0)
         self.scale = float(a["scale"]) if a.get("scale") is not None else (self.dn + self.dr) ** -0.5
         self.eps = float(a.get("eps", 1e-6))
-        if min(self.nh, self.dn, self.dv, self.rank) <= 0 or self.dr <= 0 or self.dr % 2:
+        if min(self.nh, self.dn, self.dv, self.rank) <= 0 or self.dr <= 0 or self.dr % 2 or self.q_rank < 0:
             raise ValueError("latent attention: sizes must be positive and the rotated size even")
         self.position = build_part("position", a["position"], rt)
         if int(getattr(self.position, "rotary_dim", self.dr)) != self.dr:
             raise ValueError("latent attention: the position encoding must rotate the whole rotated part")
-        self.names = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "o": "o",
-                      **(a.get("names") or {})}
+        self.half_split = getattr(self.position, "layout", "pairs") == "half"
+        self.names = {"q": "q", "q_down": "dq", "q_down_norm": "dq.norm", "q_up": "uq", "down": "dkv", "down_norm": "dkv.norm",
+                      "up_k": "uk", "up_v": "uv", "gate": "g", "o": "o", **(a.get("names") or {})}
         self.n_q = self.nh * (self.dn + self.dr)
-        self.q_down = self.out = self.wc = self.to_latent = self.from_latent = None
+        self.q_down = self.q_up = self.out = self.wc = self.wq = self.to_latent = self.from_latent = None
 
     @property
     def graph_safe(self):
@@ -145,18 +152,32 @@ class LatentAttention(Mixer):
 
     def expected_params(self):
         p, n = self.prefix, self.names
-        return {p + n["q"]: ParamSpec((self.n_q, self.hidden)),
-                p + n["down"]: ParamSpec((self.rank + self.dr, self.hidden)),
-                p + n["down_norm"]: ParamSpec((self.rank,), init="one_plus_normal"),
-                p + n["up_k"]: ParamSpec((self.nh * self.dn, self.rank)),
-                p + n["up_v"]: ParamSpec((self.nh * self.dv, self.rank)),
-                p + n["o"]: ParamSpec((self.hidden, self.nh * self.dv))}
+        e = {p + n["down"]: ParamSpec((self.rank + self.dr, self.hidden)),
+             p + n["down_norm"]: ParamSpec((self.rank,), init="one_plus_normal"),
+             p + n["up_k"]: ParamSpec((self.nh * self.dn, self.rank)),
+             p + n["up_v"]: ParamSpec((self.nh * self.dv, self.rank)),
+             p + n["o"]: ParamSpec((self.hidden, self.nh * self.dv))}
+        if self.q_rank:
+            e[p + n["q_down"]] = ParamSpec((self.q_rank, self.hidden))
+            e[p + n["q_down_norm"]] = ParamSpec((self.q_rank,), init="one_plus_normal")
+            e[p + n["q_up"]] = ParamSpec((self.n_q, self.q_rank))
+        else:
+            e[p + n["q"]] = ParamSpec((self.n_q, self.hidden))
+        if self.head_gate:
+            e[p + n["gate"]] = ParamSpec((self.nh, self.hidden))
+        return e
 
     def load_params(self, get):
         p, n = self.prefix, self.names
-        wq, wd = get(p + n["q"]), get(p + n["down"])
-        dt = torch.float32 if torch.float32 in (wq.dtype, wd.dtype) else wq.dtype
-        self.q_down = Linear(self.rt, torch.cat([wq.to(dt), wd.to(dt)], dim=0))
+        # ONE product of the mixer's input: [queries, or their latent | latent and shared key part | gates]
+        first = [get(p + n["q_down"] if self.q_rank else p + n["q"]), get(p + n["down"])]
+        if self.head_gate:
+            first.append(get(p + n["gate"]))
+        dt = torch.float32 if any(w.dtype is torch.float32 for w in first) else first[0].dtype
+        self.q_down = Linear(self.rt, torch.cat([w.to(dt) for w in first], dim=0))
+        if self.q_rank:
+            self.wq = self.rt.vector(get(p + n["q_down_norm"]))
+            self.q_up = Linear(self.rt, get(p + n["q_up"]))
         self.wc = self.rt.vector(get(p + n["down_norm"]))
         # per head: queries into the latent space (Wuk_h^T, [rank, dn]) and the summed latent out of it (Wuv_h, [dv, rank])
         uk = get(p + n["up_k"]).reshape(self.nh, self.dn, self.rank).transpose(1, 2).contiguous()
@@ -166,21 +187,36 @@ class LatentAttention(Mixer):
 
     def forward(self, xn, residual, ctx, cache):
         t, nh, dn, dr, rank = xn.shape[0], self.nh, self.dn, self.dr, self.rank
-        qd = ctx.ws.buffer("latent.qd32", (t, self.n_q + rank + dr), torch.float32)
+        n_first = self.q_rank or self.n_q
+        qd = ctx.ws.buffer("latent.qd32", (t, n_first + rank + dr + (nh if self.head_gate else 0)), torch.float32)
         self.q_down(xn, qd, ws=ctx.ws)
         cos, sin = self.position.tables(ctx)
         rows = cache.tensors["latent"]
+        slots = ctx.slot_map(cache.group) if cache.owned else None
         qfull = ctx.ws.buffer("latent.q", (t, nh, rank + dr), torch.float32)
-        ops.latent_norm_pairs_store(qd, nh, dn, dr, rank, self.wc, self.eps, cos, sin,
-                                    ctx.slot_map(cache.group) if cache.owned else None,
-                                    rows if cache.owned else None, qfull)
-        ops.headwise_linear(qd, qd.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
+        down = qd[:, n_first:n_first + rank + dr]
+        if self.q_rank:
+            # the norm of the queries' latent, the norm of the keys' latent, the rotation of the shared key part and the
+            # page write: one kernel; then the queries themselves, and the rotation of their rotated parts
+            cq = ctx.ws.buffer("latent.cq", (t, self.q_rank), self.rt.dtype)
+            ops.latent_norm_pairs_store(None, 0, dn, dr, rank, self.wc, self.eps, cos, sin, slots, rows if cache.owned else None,
+                                        None, down=down, half_split=self.half_split, q_latent=qd[:, :self.q_rank], wq=self.wq, cq=cq)
+            q = ctx.ws.buffer("latent.q32", (t, self.n_q), torch.float32)
+            self.q_up(cq, q, ws=ctx.ws)
+            ops.latent_norm_pairs_store(q, nh, dn, dr, rank, self.wc, self.eps, cos, sin, None, None, qfull, down=down,
+                                        half_split=self.half_split)
+        else:
+            q = qd
+            ops.latent_norm_pairs_store(qd, nh, dn, dr, rank, self.wc, self.eps, cos, sin, slots, rows if cache.owned else None,
+                                        qfull, half_split=self.half_split)
+        ops.headwise_linear(q, q.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
         summed = ctx.ws.buffer("latent.summed", (t, nh * rank), self.rt.dtype)
         ops.masked_attention(qfull, nh * (rank + dr), rank + dr, summed, rows, rows, ctx.attention_meta(cache.group),
                              nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale,
                              ws=ctx.ws)
         heads = ctx.ws.buffer("attn.out", (t, nh * self.dv), self.rt.dtype)
-        ops.headwise_linear(summed, nh * rank, rank, self.from_latent, heads, nh * self.dv, self.dv, t)
+        gate = qd[:, n_first + rank + dr:] if self.head_gate else None
+        ops.headwise_linear(summed, nh * rank, rank, self.from_latent, heads, nh * self.dv, self.dv, t, gate=gate)
         residual.add_linear(self.out, heads)
 
 

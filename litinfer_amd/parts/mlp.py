@@ -98,3 +98,45 @@ class ReluSquaredMLP(FeedForward):
 
 
 register_part("feed_forward", "relu2_mlp", ReluSquaredMLP)
+
+
+class GeluMLP(FeedForward):
+    """Dense feed-forward with the tanh form of GELU and biases on both products:
+    y = gelu_tanh(xn Wu^T + bu) Wd^T + bd.  The first product is left in float32 and the activation rounds once."""
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.hidden = int(spec.args["hidden_size"])
+        self.inter = int(spec.args["intermediate_size"])
+        self.biases = bool(spec.args.get("biases", True))
+        self.names = {"up": "up", "down": "down", "bias_suffix": ".b", **(spec.args.get("names") or {})}
+        self.up = None
+        self.down = None
+
+    def expected_params(self):
+        p, n = self.prefix, self.names
+        e = {p + n["up"]: ParamSpec((self.inter, self.hidden)), p + n["down"]: ParamSpec((self.hidden, self.inter))}
+        if self.biases:
+            e[p + n["up"] + n["bias_suffix"]] = ParamSpec((self.inter,), init="normal")
+            e[p + n["down"] + n["bias_suffix"]] = ParamSpec((self.hidden,), init="normal")
+        return e
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.down.row_tile() if self.down is not None else 1)
+
+    def load_params(self, get):
+        p, n = self.prefix, self.names
+        self.up = Linear(self.rt, get(p + n["up"]), get(p + n["up"] + n["bias_suffix"]) if self.biases else None)
+        self.down = Linear(self.rt, get(p + n["down"]), get(p + n["down"] + n["bias_suffix"]) if self.biases else None)
+
+    def forward(self, xn, residual, ctx):
+        t = xn.shape[0]
+        u = ctx.ws.buffer("mlp.up32", (t, self.inter), torch.float32)
+        self.up(xn, u, ws=ctx.ws)
+        h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)
+        ops.gelu_tanh(u, h)
+        residual.add_linear(self.down, h)
+
+
+register_part("feed_forward", "gelu_mlp", GeluMLP)

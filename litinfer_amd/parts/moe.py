@@ -1,16 +1,23 @@
 """A routed feed-forward: `experts` small feed-forwards of which every token uses `top`, and an optional shared
 one that every token uses.
 
-Router: logits = xn Wr^T + br in float32; the `top` largest are chosen (the lower index wins a tie) and weighted
-by the softmax over the chosen logits alone.  An expert is Wdown act(Wup xn) with act = max(., 0)^2, no biases.
-The shared expert has the same form with a width of its own; its output is multiplied by sigmoid(wg . xn), one
+Router: logits = xn Wr^T (+ br) in float32.  `scores` = "softmax_chosen": the `top` largest logits are chosen (the
+lower index wins a tie) and weighted by the softmax over the chosen logits alone.  `scores` = "sigmoid": an
+expert's score is sigmoid(logit); the choice goes by score + correction (a stored vector, one number an expert,
+that the weights do not see), and, where the experts form `groups` groups of neighbours, only among the experts of
+the `keep_groups` groups whose two largest choice values have the largest sum; the weights are the chosen scores
+divided by their sum.
+An expert (`activation`): "relu2" is Wdown max(Wup xn, 0)^2; "swiglu" is Wdown (silu(Wgate xn) * (Wup xn)).  No
+biases.  The shared expert (relu2 only) has a width of its own; its output is multiplied by sigmoid(wg . xn), one
 number a token, where a gate row is given.  The output is the weighted sum, added to the stream in float32.
 
 On the device: one kernel routes (logits, choice, weights and the shared gate), one sorts the step's (token,
 choice) pairs by expert and cuts them into tiles of rows, the two products run tile by tile against the
-tile's expert (the activation is the first one's epilogue), and one kernel adds the weighted rows and the gated
+tile's expert (the squared ReLU is the first one's epilogue; gate and up are ONE product whose float32 result the
+activation kernel reads), and one kernel adds the weighted rows and the gated
 shared output into the stream, in the order of the choices.  No number returns to the host, so a decoding step
-can be recorded.  The experts' matrices are bound as two tensors [experts, ff, hidden] and [experts, hidden, ff].
+can be recorded.  The experts' matrices are bound as two tensors [experts, ff (or 2 ff: gates, then ups), hidden]
+and [experts, hidden, ff].
 """
 from __future__ import annotations
 
@@ -22,8 +29,9 @@ from .base import BatchNeeds, FeedForward, register_part
 from .linear import Linear
 
 
-class RoutedReluSquaredMLP(FeedForward):
+class RoutedMLP(FeedForward):
     graph_safe = True
+    default_activation = "swiglu"
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -32,24 +40,47 @@ class RoutedReluSquaredMLP(FeedForward):
         self.experts = int(a["experts"])
         self.top = int(a["top"])
         self.inter = int(a["intermediate_size"])
+        self.activation = str(a.get("activation") or self.default_activation)
+        self.scores = str(a.get("scores") or "softmax_chosen")
+        self.groups = int(a.get("groups") or 1)
+        self.keep_groups = int(a.get("keep_groups") or self.groups)
+        self.has_correction = bool(a.get("correction", False))
+        self.has_router_bias = bool(a.get("router_bias", self.scores == "softmax_chosen"))
         self.shared_inter = int(a.get("shared_intermediate_size") or 0)
         self.shared_gate = bool(a.get("shared_gate", True)) and self.shared_inter > 0
         if min(self.hidden, self.experts, self.top, self.inter) <= 0 or self.top > self.experts:
             raise ValueError(f"routed feed-forward: {self.top} of {self.experts} experts of width {self.inter}")
         if self.top > 64:
             raise ValueError("routed feed-forward: the router kernel picks at most 64 experts a token")
-        self.names = {"expert": "e{}.", "up": "up", "down": "down", "router": "router", "router_bias": "router.b",
-                      "shared": "shared.", "shared_gate": "sg", **(a.get("names") or {})}
-        self.w_up = self.w_down = self.router = self.router_b = self.gate_row = self.shared_up = self.shared_down = None
+        if self.activation not in ("relu2", "swiglu") or self.scores not in ("softmax_chosen", "sigmoid"):
+            raise ValueError(f"routed feed-forward: activation {self.activation!r}, scores {self.scores!r}")
+        if self.scores != "sigmoid" and (self.groups != 1 or self.has_correction):
+            raise ValueError("routed feed-forward: groups and a correction of the choice belong to sigmoid scores")
+        if not 1 <= self.keep_groups <= self.groups or self.experts % self.groups:
+            raise ValueError(f"routed feed-forward: {self.experts} experts in {self.groups} groups of which {self.keep_groups} are kept")
+        if self.top > self.keep_groups * (self.experts // self.groups):
+            raise ValueError(f"routed feed-forward: {self.top} choices, but the kept groups hold "
+                             f"{self.keep_groups * (self.experts // self.groups)} experts")
+        if self.shared_inter and self.activation != "relu2":
+            raise ValueError("routed feed-forward: the shared expert is a squared-ReLU one")
+        self.names = {"expert": "e{}.", "up": "up", "gate": "gate", "down": "down", "router": "router", "router_bias": "router.b",
+                      "correction": "correction", "shared": "shared.", "shared_gate": "sg", **(a.get("names") or {})}
+        self.w_up = self.w_down = self.router = self.router_b = self.correction = None
+        self.gate_row = self.shared_up = self.shared_down = None
 
     def _expert(self, e: int, which: str) -> str:
         return self.prefix + self.names["expert"].format(e) + self.names[which]
 
     def expected_params(self):
         p, n = self.prefix, self.names
-        out = {p + n["router"]: ParamSpec((self.experts, self.hidden)),
-               p + n["router_bias"]: ParamSpec((self.experts,), init="zeros")}
+        out = {p + n["router"]: ParamSpec((self.experts, self.hidden))}
+        if self.has_router_bias:
+            out[p + n["router_bias"]] = ParamSpec((self.experts,), init="zeros")
+        if self.has_correction:
+            out[p + n["correction"]] = ParamSpec((self.experts,), init="normal")
         for e in range(self.experts):
+            if self.activation == "swiglu":
+                out[self._expert(e, "gate")] = ParamSpec((self.inter, self.hidden))
             out[self._expert(e, "up")] = ParamSpec((self.inter, self.hidden))
             out[self._expert(e, "down")] = ParamSpec((self.hidden, self.inter))
         if self.shared_inter:
@@ -65,10 +96,15 @@ class RoutedReluSquaredMLP(FeedForward):
 
     def load_params(self, get):
         p, n = self.prefix, self.names
-        self.w_up = self.rt.matrix(torch.stack([get(self._expert(e, "up")) for e in range(self.experts)]))
+        if self.activation == "swiglu":      # an expert's gates, then its ups: one product
+            first = [torch.cat([get(self._expert(e, "gate")), get(self._expert(e, "up"))], dim=0) for e in range(self.experts)]
+        else:
+            first = [get(self._expert(e, "up")) for e in range(self.experts)]
+        self.w_up = self.rt.matrix(torch.stack(first))
         self.w_down = self.rt.matrix(torch.stack([get(self._expert(e, "down")) for e in range(self.experts)]))
         self.router = self.rt.matrix(get(p + n["router"]))
-        self.router_b = self.rt.vector(get(p + n["router_bias"]))
+        self.router_b = self.rt.vector(get(p + n["router_bias"])) if self.has_router_bias else None
+        self.correction = self.rt.vector(get(p + n["correction"])) if self.has_correction else None
         if self.shared_inter:
             s = p + n["shared"]
             self.shared_up = Linear(self.rt, get(s + n["up"]))
@@ -82,17 +118,24 @@ class RoutedReluSquaredMLP(FeedForward):
         idx = ws.buffer("moe.idx", (t, top), torch.int32)
         wt = ws.buffer("moe.wt", (t, top), torch.float32)
         gate = ws.buffer("moe.gate", (t,), torch.float32) if self.gate_row is not None else None
-        ops.moe_route(xn, self.router, self.router_b, self.gate_row, idx, wt, gate)
+        ops.moe_route(xn, self.router, self.router_b, self.gate_row, idx, wt, gate, scores=self.scores,
+                      correction=self.correction, groups=self.groups, keep_groups=self.keep_groups)
         # (a prompt's portion gives every expert hundreds of rows: larger tiles then, for the kernel that stages them in LDS)
+        n_first = self.w_up.shape[1]
         rows_a_tile = ops.moe_tile_rows(t, top, self.experts, xn.dtype, self.w_up.dtype,
-                                        ((self.inter, self.hidden), (self.hidden, self.inter)))
+                                        ((n_first, self.hidden), (self.hidden, self.inter)))
         max_tiles = ops.moe_max_tiles(t, top, self.experts, rows_a_tile)
         plan = ws.buffer("moe.plan", (4 + 4 * max_tiles,), torch.int32)
         row_token = ws.buffer("moe.row_token", (pairs,), torch.int32)
         pair_row = ws.buffer("moe.pair_row", (pairs,), torch.int32)
         ops.moe_plan(idx, self.experts, plan, row_token, pair_row, rows_a_tile)
         h = ws.buffer("moe.h", (pairs, self.inter), self.rt.dtype)
-        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1, tile_rows=rows_a_tile)
+        if self.activation == "swiglu":
+            gu = ws.buffer("moe.gate_up32", (pairs, n_first), torch.float32)
+            ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, gu, pairs, tile_rows=rows_a_tile)
+            ops.swiglu_rows(gu, h)
+        else:
+            ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1, tile_rows=rows_a_tile)
         yrows = ws.buffer("moe.y", (pairs, self.hidden), torch.float32)
         ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs, tile_rows=rows_a_tile)
         shared = None
@@ -106,4 +149,10 @@ class RoutedReluSquaredMLP(FeedForward):
         ops.moe_combine(residual.tensor(), yrows, pair_row, wt, gate, shared)
 
 
+class RoutedReluSquaredMLP(RoutedMLP):
+    """Squared-ReLU experts behind a router with bias and a softmax over the chosen logits, plus a gated shared expert."""
+    default_activation = "relu2"
+
+
 register_part("feed_forward", "routed_relu2", RoutedReluSquaredMLP)
+register_part("feed_forward", "routed_mlp", RoutedMLP)

@@ -117,7 +117,8 @@ class RopePairs(Position):
     (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rotary_dim - 1) and
     ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency is f_i / factor * ramp_i +
     f_i (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1.  The frequencies are
-    worked out once on the host (float64, rounded to float32); the angle, cos and sin are float32."""
+    worked out once on the host (float64, rounded to float32); the angle, cos and sin are float32.
+    With layout "half" the same angles rotate column i with column i + rotary_dim/2 instead."""
     graph_safe = True
 
     def __init__(self, spec, rt):
@@ -127,6 +128,10 @@ class RopePairs(Position):
         self.rotary_dim = int(a.get("rotary_dim", self.head_dim))
         self.theta = float(a["theta"])
         self.scaling = dict(a["scaling"]) if a.get("scaling") else None
+        # which columns form a pair: "pairs" (2i, 2i + 1) or "half" (i, i + rotary_dim / 2); the angles are the same
+        self.layout = str(a.get("layout") or "pairs")
+        if self.layout not in ("pairs", "half"):
+            raise ValueError(f"rope: layout must be 'pairs' or 'half', found {self.layout!r}")
         if self.theta <= 0:
             raise ValueError(f"rope: theta must be positive, found {self.theta}")
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
@@ -154,7 +159,10 @@ class RopePairs(Position):
 
     def apply(self, qkv, n_heads_total, head_dim, ctx):
         cos, sin = self.tables(ctx)
-        ops.rope_pairs_apply(qkv, n_heads_total, head_dim, self.rotary_dim, cos, sin)
+        if self.layout == "half":
+            ops.rope_apply(qkv, n_heads_total, head_dim, self.rotary_dim, cos, sin)
+        else:
+            ops.rope_pairs_apply(qkv, n_heads_total, head_dim, self.rotary_dim, cos, sin)
 
 
 def pair_frequencies(rotary_dim: int, theta: float, scaling=None):
