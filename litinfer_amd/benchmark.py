@@ -760,9 +760,43 @@ def sogenex_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, obje
             "logit_softcap": 30.0, "layers": [attn if i % 3 == 1 else ssm for i in range(layers)]}
 
 
+NUSUVIK_SIZES = {         # queries' latent; experts, chosen, groups, kept groups, expert width (the chosen gated experts together
+    # hold about as many weights as the dense feed-forward)
+    "1.5b": (768, 16, 4, 4, 2, 1536),
+    "7b": (1536, 16, 4, 4, 2, 3200),
+}
+
+
+def nusuvik_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, object]:
+    """A Nusuvik model at the layer sizes of a Qwen2 family member: attention over a compressed cache in every layer
+    (no window), a dense and a routed feed-forward in turn, layers 1..2 passed twice, a hashed pair table."""
+    width, heads, _, dim, ff, rank, rot, _ = DESIGN_SIZES[size]
+    q_rank, ne, top, groups, keep, eff = NUSUVIK_SIZES[size]
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": rank, "q_rank": q_rank,
+             "scale": (dim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": ne, "top": top, "groups": {"count": groups, "keep": keep}}}
+    return {"architecture": "Nusuvik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "embedding": {"bigram": {"buckets": 100003, "mul_prev": 36313, "mul_cur": 27191}},
+            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe} for i in range(layers)],
+            "loop": {"start": 1, "stop": 3, "times": 2} if layers >= 4 else None}
+
+
+def tovasun_latent_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, object]:
+    """The closest existing model to Nusuvik: a Tovasun model whose every layer is attention over a compressed cache of
+    the same sizes, without window and token input, with dense feed-forwards and the same loop."""
+    width, heads, _, dim, ff, rank, rot, _ = DESIGN_SIZES[size]
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+              "mixer": {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+                        "rot": {"base": 10000.0, "dims": rot}}}
+    return {"architecture": "Tovasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": [latent] * layers,
+            "loop": {"start": 1, "stop": 3, "times": 2} if layers >= 4 else None}
+
+
 def compare_designs(a) -> Dict[str, object]:
-    """Prefill and decode throughput of a second design (`--design`: Tovasun or Sogenex) beside Qwen2 at the same
-    width, heads, (active) feed-forward width, window and number of layer runs (random weights, random cache content)."""
+    """Prefill and decode throughput of a second design (`--design`: Tovasun, Sogenex or Nusuvik) beside Qwen2 (Nusuvik:
+    beside its closest relative, an all-latent Tovasun model) at the same width, heads, (active) feed-forward width,
+    window and number of layer runs (random weights, random cache content)."""
     import numpy as np
     import torch
     from .engine import Engine, StepEntry
@@ -773,15 +807,20 @@ def compare_designs(a) -> Dict[str, object]:
     for size in sizes:
         layers = a.layers or 6
         design = getattr(a, "design", None) or "tovasun"
-        tcfg = sogenex_config(size, layers) if design == "sogenex" else tovasun_config(size, layers)
+        tcfg = {"sogenex": sogenex_config, "nusuvik": nusuvik_config}.get(design, tovasun_config)(size, layers)
         runs = layers + (2 if tcfg.get("loop") else 0)
         width, heads, kv, dim, ff = DESIGN_SIZES[size][:5]
-        qcfg = dict(SHAPES[size], num_hidden_layers=runs, vocab_size=32000, use_sliding_window=True,
-                    sliding_window=DESIGN_WINDOW, max_window_layers=0, max_position_embeddings=8192)
+        if design == "nusuvik":
+            beside, qcfg = "tovasun", tovasun_latent_config(size, layers)
+        else:
+            beside = "qwen2"
+            qcfg = dict(SHAPES[size], num_hidden_layers=runs, vocab_size=32000, use_sliding_window=True,
+                        sliding_window=DESIGN_WINDOW, max_window_layers=0, max_position_embeddings=8192)
         res = {}
-        for name, cfg, vocab in ((design, tcfg, tcfg["vocab"]), ("qwen2", qcfg, qcfg["vocab_size"])):
+        for name, cfg, vocab in ((design, tcfg, tcfg["vocab"]), (beside, qcfg, 32000)):
             eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
-                                     num_pages=(64 * (DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE, max_seqs=65)
+                                     num_pages=(64 * ((2 if design == "nusuvik" else 1) * DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE,
+                                     max_seqs=65)
             for g in eng.cache.groups:
                 for data in g.data.values():
                     data.normal_(0, 0.5)
@@ -827,17 +866,18 @@ def compare_designs(a) -> Dict[str, object]:
             log(f"{size} {name}: {r}")
             del eng
             torch.cuda.empty_cache()
-        res[f"{design}_over_qwen2"] = {k: round(res[design][k] / res["qwen2"][k], 3)
-                                       for k in res["qwen2"] if k.endswith("tok_s")}
+        res[f"{design}_over_{beside}"] = {k: round(res[design][k] / res[beside][k], 3)
+                                          for k in res[beside] if k.endswith("tok_s")}
         out[size] = res
     first = out[sizes[0]]
     title = design.capitalize()
-    return {"metric": f"decode tok/s ({title} at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, window {DESIGN_WINDOW})",
+    return {"metric": f"decode tok/s ({title} at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, "
+                      + ("no window)" if design == "nusuvik" else f"window {DESIGN_WINDOW})"),
             "value": first[design][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
             "warmup": a.warmup, "ms_per_step": first[design][f"decode_b{a.batch}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
             "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content",
-            "config": {"model": f"{title} beside Qwen2 at equal layer sizes", "global_batch": a.batch,
+            "config": {"model": f"{title} beside {beside.capitalize()} at equal layer sizes", "global_batch": a.batch,
                        "seq_len": 2 * DESIGN_WINDOW, "prefill_tokens": PREFILL_TOKENS, "page_size": PAGE,
                        "parallelism": "none (1 GPU)"},
             "designs": out}
@@ -854,7 +894,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep", "designs"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="sweep: the member of the family whose layer sizes are taken (7b); designs: 1.5b or 7b (both)")
-    ap.add_argument("--design", default="tovasun", choices=["tovasun", "sogenex"],
+    ap.add_argument("--design", default="tovasun", choices=["tovasun", "sogenex", "nusuvik"],
                     help="designs: the design that is set beside Qwen2")
     ap.add_argument("--page-order-seed", type=int, default=0,
                     help="headline: the cache's pages are handed out in a shuffled order, as a pool that has served requests "

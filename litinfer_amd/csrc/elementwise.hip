@@ -995,23 +995,3 @@ extern "C" int li_concat_rows(const float* a, const float* b, void* out, int out
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }
-
-// out[r, i] = silu(gu[r, i]) * gu[r, I + i] for float32 rows of gate and up values, in the dtype of out
-template <typename TO>
-__global__ void swiglu_rows_kernel(const float* __restrict__ gu, TO* __restrict__ out, long rows, int I) {
-    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= rows * I) return;
-    const long r = idx / I;
-    const int i = (int)(idx % I);
-    const float g = gu[r * 2 * I + i], u = gu[r * 2 * I + I + i];
-    store_from_float(out + idx, u * (g / (1.0f + expf(-g))));
-}
-
-extern "C" int li_swiglu_rows(const float* gu, void* out, int out_dtype, long rows, int I, hipStream_t stream) {
-    if (rows <= 0 || I <= 0) return LI_ERR_SIZE;
-    const unsigned blocks = (unsigned)((rows * I + 255) / 256);
-    if (out_dtype == LI_F32) swiglu_rows_kernel<float><<<blocks, 256, 0, stream>>>(gu, (float*)out, rows, I);
-    else if (out_dtype == LI_BF16) swiglu_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gu, (bf16_t*)out, rows, I);
-    else return LI_ERR_DTYPE;
-    return li_launch_status();
-}

@@ -219,9 +219,35 @@ extern "C" int li_moe_plan(const int* idx, int T, int top, int E, int* plan, int
     return li_launch_status();
 }
 
+// Four consecutive outputs of one row, from column `col` (a multiple of 4) on, with the activation: 0 none, 1 max(., 0)^2,
+// 2 the columns are (gate, up) pairs and the two results silu(gate) * up go to columns col / 2 and col / 2 + 1.
+template <typename TO>
+__device__ __forceinline__ void moe_store4(TO* __restrict__ row, int col, float v0, float v1, float v2, float v3, int act) {
+    if (act == 2) {
+        const float o0 = v1 * (v0 / (1.0f + expf(-v0))), o1 = v3 * (v2 / (1.0f + expf(-v2)));
+        TO* dst = row + (col >> 1);
+        if constexpr (sizeof(TO) == 2) *reinterpret_cast<uint32_t*>(dst) = pack2_bf16(o0, o1);
+        else *reinterpret_cast<float2*>(dst) = float2{o0, o1};
+        return;
+    }
+    if (act == 1) {
+        v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); v2 = fmaxf(v2, 0.f); v3 = fmaxf(v3, 0.f);
+        v0 *= v0; v1 *= v1; v2 *= v2; v3 *= v3;
+    }
+    TO* dst = row + col;
+    if constexpr (sizeof(TO) == 2) {
+        uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+        d2[0] = pack2_bf16(v0, v1);
+        d2[1] = pack2_bf16(v2, v3);
+    } else {
+        *reinterpret_cast<float4*>(dst) = float4{v0, v1, v2, v3};
+    }
+}
+
 // ---------------------------------------------------------------------------------------- products by tile
 // out[row, j] = act(sum_k W[e, j, k] * a[src(row), k]) for the rows of every tile, e the tile's expert; src(row) =
-// row_token[row] where the rows are gathered from tokens, else the row itself.  act: 0 none, 1 max(., 0)^2.
+// row_token[row] where the rows are gathered from tokens, else the row itself.  act: 0 none, 1 max(., 0)^2, 2 the
+// matrix rows come in pairs (2 j: gate, 2 j + 1: up) and out[row, j] = silu(gate) * up: half as many columns.
 // General form: a block takes a tile and 64 outputs; rows and matrix rows go through LDS in float32, K in steps
 // of 32; a thread owns 2 rows x 4 outputs.  Sums are float32 in the order of k.
 template <typename TA, typename TW, typename TO>
@@ -239,7 +265,7 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ 
         const int r = r0 + (threadIdx.x < nr ? threadIdx.x : 0);
         src[threadIdx.x] = row_token ? row_token[r] : r;
     }
-    const int tr = threadIdx.x / 16, tc = threadIdx.x % 16;          // rows 2 tr, 2 tr + 1; outputs tc + 16 i
+    const int tr = threadIdx.x / 16, tc = threadIdx.x % 16;          // rows 2 tr, 2 tr + 1; outputs 2 tc + (i & 1) + 32 (i >> 1)
     float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     const TW* we = w + (size_t)e * n_out * K;
     for (int k0 = 0; k0 < K; k0 += 32) {
@@ -258,7 +284,7 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ 
             const float a0 = As[2 * tr][k], a1 = As[2 * tr + 1][k];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float wv = Ws[tc + 16 * i][k];
+                const float wv = Ws[2 * tc + (i & 1) + 32 * (i >> 1)][k];
                 acc[0][i] = fmaf(a0, wv, acc[0][i]);
                 acc[1][i] = fmaf(a1, wv, acc[1][i]);
             }
@@ -270,9 +296,14 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ 
         if (r >= nr) continue;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int j = j0 + tc + 16 * i;
+            const int j = j0 + 2 * tc + (i & 1) + 32 * (i >> 1);
             if (j >= n_out) continue;
             float v = acc[rr][i];
+            if (act == 2) {                            // (gate, up) pairs: i even holds the gate, i + 1 the up value
+                if (i & 1) continue;
+                store_from_float(out + (size_t)(r0 + r) * out_stride + (j >> 1), acc[rr][i + 1] * (v / (1.0f + expf(-v))));
+                continue;
+            }
             if (act == 1) { v = fmaxf(v, 0.f); v = v * v; }
             store_from_float(out + (size_t)(r0 + r) * out_stride + j, v);
         }
@@ -317,24 +348,10 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const TA* __restri
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, fb.v, acc, 0, 0, 0);
     }
     if (ql >= nr) return;
-    TO* orow = out + (size_t)(r0 + ql) * out_stride + j0;
+    TO* orow = out + (size_t)(r0 + ql) * out_stride;
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {                   // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[i] = acc[4 * rg + i];
-            if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
-        }
-        TO* dst = orow + 8 * rg + 4 * h2;
-        if constexpr (sizeof(TO) == 2) {
-            uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
-            d2[0] = pack2_bf16(v[0], v[1]);
-            d2[1] = pack2_bf16(v[2], v[3]);
-        } else {
-            *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
-        }
-    }
+    for (int rg = 0; rg < 4; ++rg)                     // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
+        moe_store4(orow, j0 + 8 * rg + 4 * h2, acc[4 * rg], acc[4 * rg + 1], acc[4 * rg + 2], acc[4 * rg + 3], act);
 }
 
 // The wider form, for K a multiple of 32: a wave takes the tile's 32 rows and 128 outputs (four accumulators that
@@ -442,26 +459,12 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
         f_hi = wv + 1;
     }
     if (ql >= nr) return;
-    TO* orow = out + (size_t)(r0 + ql) * out_stride + j0;
+    TO* orow = out + (size_t)(r0 + ql) * out_stride;
     for (int f = f_lo; f < f_hi; ++f) {
         const moe_f32x16 c = KSPLIT > 1 ? acc[0] : (f == 0 ? acc[0] : f == 1 ? acc[1] : f == 2 ? acc[2] : acc[3]);
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 32 f + 8 rg + 4 h2 ..
-            float v[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                v[i] = c[4 * rg + i];
-                if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
-            }
-            TO* dst = orow + 32 * f + 8 * rg + 4 * h2;
-            if constexpr (sizeof(TO) == 2) {
-                uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
-                d2[0] = pack2_bf16(v[0], v[1]);
-                d2[1] = pack2_bf16(v[2], v[3]);
-            } else {
-                *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
-            }
-        }
+        for (int rg = 0; rg < 4; ++rg)                 // registers 4 rg .. 4 rg + 3: outputs 32 f + 8 rg + 4 h2 ..
+            moe_store4(orow, j0 + 32 * f + 8 * rg + 4 * h2, c[4 * rg], c[4 * rg + 1], c[4 * rg + 2], c[4 * rg + 3], act);
     }
 }
 
@@ -529,12 +532,22 @@ __global__ __launch_bounds__(256) void moe_linear_rows_kernel(const bf16_t* __re
 #pragma unroll
             for (int r = 0; r < MR_ROWS; ++r) {
                 if (rc + r >= nr) continue;
+                TO* orow = out + (size_t)(r0 + rc + r) * out_stride;
+                if (act == 2) {                        // (gate, up) pairs: n_out is even and j0 a multiple of 4
+#pragma unroll
+                    for (int j = 0; j < MR_OUT; j += 2)
+                        if (j0 + j < n_out) {
+                            const float g = acc[j][r];
+                            store_from_float(orow + ((j0 + j) >> 1), acc[j + 1][r] * (g / (1.0f + expf(-g))));
+                        }
+                    continue;
+                }
 #pragma unroll
                 for (int j = 0; j < MR_OUT; ++j) {
                     if (j0 + j >= n_out) continue;
                     float v = acc[j][r];
                     if (act == 1) { v = fmaxf(v, 0.f); v = v * v; }
-                    store_from_float(out + (size_t)(r0 + rc + r) * out_stride + j0 + j, v);
+                    store_from_float(orow + j0 + j, v);
                 }
             }
         }
@@ -651,27 +664,14 @@ __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __res
     for (int rf = 0; rf < RF; ++rf) {
         const int row = 32 * RF * wr + 32 * rf + ql;
         if (row >= nr) continue;
-        TO* orow = out + (size_t)(r0 + row) * out_stride + j0 + 64 * wc;
+        TO* orow = out + (size_t)(r0 + row) * out_stride;
 #pragma unroll
         for (int cf = 0; cf < 2; ++cf) {
             if (j0 + 64 * wc + 32 * cf >= n_out) continue;
 #pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {           // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
-                float v[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    v[i] = acc[rf][cf][4 * rg + i];
-                    if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
-                }
-                TO* dst = orow + 32 * cf + 8 * rg + 4 * h2;
-                if constexpr (sizeof(TO) == 2) {
-                    uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
-                    d2[0] = pack2_bf16(v[0], v[1]);
-                    d2[1] = pack2_bf16(v[2], v[3]);
-                } else {
-                    *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
-                }
-            }
+            for (int rg = 0; rg < 4; ++rg)             // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
+                moe_store4(orow, j0 + 64 * wc + 32 * cf + 8 * rg + 4 * h2, acc[rf][cf][4 * rg], acc[rf][cf][4 * rg + 1],
+                           acc[rf][cf][4 * rg + 2], acc[rf][cf][4 * rg + 3], act);
         }
     }
 }
@@ -684,7 +684,9 @@ extern "C" int li_moe_linear_big_takes(int a_dtype, int w_dtype, int n_out, int 
 extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
                              const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
                              int tile_rows, int rows, hipStream_t stream) {
-    if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
+    if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || act < 0 || act > 2 || out_stride < (act == 2 ? n_out / 2 : n_out) ||
+        (act == 2 && (n_out & 1)))
+        return LI_ERR_SIZE;
     if (tile_rows == MOE_BIG_TILE || tile_rows == MOE_HUGE_TILE) {
         if (!li_moe_linear_big_takes(a_dtype, w_dtype, n_out, K) || a_stride % 8 || out_stride % 4 ||
             ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16)

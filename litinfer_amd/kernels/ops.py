@@ -48,7 +48,6 @@ _SIGNATURES = {
         "li_layernorm": [P, P, P, F, P, I, I, I],
         "li_gelu_tanh": [P, I, P, I, L],
         "li_concat_rows": [P, P, P, I, I, I],
-        "li_swiglu_rows": [P, P, I, L, I],
         "li_sinusoid_add": [P, P, P, I, I],
         "li_scale_softcap": [P, L, F, F],
         "li_paged_store": [P, L, I, I, I, P, I, I, I, P, I, I, I, P, I, P, I, I],
@@ -580,16 +579,6 @@ def concat_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
          and out.shape == (t, 2 * h) and out.is_contiguous() and out.dtype in _DT, "concat_rows: a, b [T, H] float32, out [T, 2H]")
     if t:
         _run("elementwise", "li_concat_rows", a.data_ptr(), b.data_ptr(), out.data_ptr(), _DT[out.dtype], t, h)
-
-
-def swiglu_rows(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[r, i] = silu(gate_up[r, i]) * gate_up[r, I + i] for float32 gate_up [R, 2I]; out [R, I] in its own dtype."""
-    _gpu(gate_up, out)
-    r, inter = out.shape
-    _chk(gate_up.shape == (r, 2 * inter) and gate_up.is_contiguous() and out.is_contiguous()
-         and gate_up.dtype is torch.float32 and out.dtype in _DT, "swiglu_rows: gate_up float32 [R, 2I], out [R, I]")
-    if r:
-        _run("elementwise", "li_swiglu_rows", gate_up.data_ptr(), out.data_ptr(), _DT[out.dtype], r, inter)
 
 
 _CUS: Dict[int, int] = {}
@@ -1602,11 +1591,14 @@ def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: tor
 def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tensor, plan: torch.Tensor, max_tiles: int,
                out: torch.Tensor, rows: int, act: int = 0, tile_rows: int = MOE_TILE_ROWS) -> None:
     """out[row] = act(W[expert of the row's tile] a[src(row)]) for the sorted rows of the plan; src(row) = row_token[row]
-    where given (rows gathered from tokens), else the row.  w [experts, n_out, K]; act 1: max(., 0)^2."""
+    where given (rows gathered from tokens), else the row.  w [experts, n_out, K]; act 1: max(., 0)^2; act 2: the
+    matrix rows are (gate, up) pairs, out[row, j] = silu(W[2j] a) * (W[2j + 1] a) and out has n_out / 2 columns."""
     _gpu(a, row_token, w, plan, out)
     e, n_out, k = w.shape
+    _chk(act in (0, 1, 2) and (act != 2 or n_out % 2 == 0), "moe_linear: act")
     _chk(a.dtype in _DT and _rows_ok(a) and a.shape[1] == k and w.dtype in _DT and w.is_contiguous() and out.dtype in _DT and _rows_ok(out)
-         and out.shape == (rows, n_out) and (w.dtype is torch.bfloat16 or (a.dtype is torch.float32 and out.dtype is torch.float32)),
+         and out.shape == (rows, n_out // 2 if act == 2 else n_out)
+         and (w.dtype is torch.bfloat16 or (a.dtype is torch.float32 and out.dtype is torch.float32)),
          "moe_linear: a [*, K], w [E, n_out, K], out [rows, n_out]")
     _chk(plan.dtype is torch.int32 and plan.numel() >= 4 + 4 * max_tiles and (row_token is not None or a.shape[0] >= rows)
          and (row_token is None or (row_token.dtype is torch.int32 and row_token.numel() >= rows)), "moe_linear: plan, rows")

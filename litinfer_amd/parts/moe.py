@@ -13,11 +13,11 @@ number a token, where a gate row is given.  The output is the weighted sum, adde
 
 On the device: one kernel routes (logits, choice, weights and the shared gate), one sorts the step's (token,
 choice) pairs by expert and cuts them into tiles of rows, the two products run tile by tile against the
-tile's expert (the squared ReLU is the first one's epilogue; gate and up are ONE product whose float32 result the
-activation kernel reads), and one kernel adds the weighted rows and the gated
-shared output into the stream, in the order of the choices.  No number returns to the host, so a decoding step
-can be recorded.  The experts' matrices are bound as two tensors [experts, ff (or 2 ff: gates, then ups), hidden]
-and [experts, hidden, ff].
+tile's expert (the activation is the first one's epilogue; gate and up are ONE product whose matrix holds an
+expert's gate and up rows in turn, so that a thread of the product ends with both factors of an output), and one
+kernel adds the weighted rows and the gated shared output into the stream, in the order of the choices.  No number
+returns to the host, so a decoding step can be recorded.  The experts' matrices are bound as two tensors
+[experts, ff (or 2 ff), hidden] and [experts, hidden, ff].
 """
 from __future__ import annotations
 
@@ -96,8 +96,9 @@ class RoutedMLP(FeedForward):
 
     def load_params(self, get):
         p, n = self.prefix, self.names
-        if self.activation == "swiglu":      # an expert's gates, then its ups: one product
-            first = [torch.cat([get(self._expert(e, "gate")), get(self._expert(e, "up"))], dim=0) for e in range(self.experts)]
+        if self.activation == "swiglu":      # an expert's gate and up rows in turn: one product, the activation its epilogue
+            first = [torch.stack([get(self._expert(e, "gate")), get(self._expert(e, "up"))], dim=1).reshape(2 * self.inter, self.hidden)
+                     for e in range(self.experts)]
         else:
             first = [get(self._expert(e, "up")) for e in range(self.experts)]
         self.w_up = self.rt.matrix(torch.stack(first))
@@ -130,12 +131,8 @@ class RoutedMLP(FeedForward):
         pair_row = ws.buffer("moe.pair_row", (pairs,), torch.int32)
         ops.moe_plan(idx, self.experts, plan, row_token, pair_row, rows_a_tile)
         h = ws.buffer("moe.h", (pairs, self.inter), self.rt.dtype)
-        if self.activation == "swiglu":
-            gu = ws.buffer("moe.gate_up32", (pairs, n_first), torch.float32)
-            ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, gu, pairs, tile_rows=rows_a_tile)
-            ops.swiglu_rows(gu, h)
-        else:
-            ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1, tile_rows=rows_a_tile)
+        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=2 if self.activation == "swiglu" else 1,
+                       tile_rows=rows_a_tile)
         yrows = ws.buffer("moe.y", (pairs, self.hidden), torch.float32)
         ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs, tile_rows=rows_a_tile)
         shared = None
