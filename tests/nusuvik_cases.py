@@ -103,3 +103,44 @@ def write_model(folder, config, weights, dtype=torch.float32):
 def stored(weights, dtype):
     """The weights as a checkpoint of `dtype` holds them, float64."""
     return {n: torch.from_numpy(a).to(dtype).to(torch.float64).numpy() for n, a in weights.items()}
+
+
+def random_config(seed):
+    """A configuration drawn from a seed: every size, the order of layers, the loop and the routers' shapes vary."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(0, len(xs)))]
+    n = int(rng.integers(2, 6))
+    width = pick(64, 72, 96, 160, 192, 256, 328, 384)
+    kinds = []
+
+    def mixer():
+        heads, dim, rot = pick(1, 2, 3, 4, 6, 8, 16), pick(8, 16, 24, 32, 64, 128), pick(2, 8, 16, 32, 64)
+        return dict(heads=heads, dim=dim, rot_dim=rot, vdim=pick(8, 16, 32, 48, 64, 128), kv_rank=pick(8, 24, 32, 64, 96, 128),
+                    q_rank=pick(8, 16, 48, 64, 128, 192), scale=float(rng.uniform(0.5, 1.5)) / np.sqrt(dim + rot),
+                    base=pick(100.0, 10000.0, 1000000.0))
+    shared = mixer()
+    layers = []
+    for i in range(n):
+        m = shared if rng.random() < 0.6 else mixer()           # (equal mixers share a page group)
+        kind = pick("dense", "moe", "moe", None)
+        if kind == "dense":
+            mlp = dense(pick(32, 100, 256, 520))
+        elif kind == "moe":
+            groups = pick(1, 2, 3, 4)
+            per = pick(1, 2, 4) if groups > 1 else pick(2, 3, 8)
+            keep = int(rng.integers(1, groups + 1))
+            top = int(rng.integers(1, min(keep * per, 6) + 1))
+            mlp = moe(groups * per, top, pick(16, 40, 64, 96), groups if rng.random() < 0.8 or groups > 1 else None, keep)
+        else:
+            mlp = None
+        kinds.append(kind)
+        layers.append(latent_layer(m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"], m["scale"], mlp, m["base"]))
+    cfg = {"architecture": "Nusuvik", "vocab": pick(61, 200, 448, 515), "width": width, "norm": {"eps": pick(1e-6, 1e-5, 1e-3)}, "layers": layers}
+    if rng.random() < 0.8:
+        cfg["embedding"] = {"bigram": {"buckets": pick(7, 509, 4099), "mul_prev": pick(1, 31, 65537), "mul_cur": pick(1, 7, 1009)}}
+    if rng.random() < 0.8:
+        start = int(rng.integers(0, n))
+        cfg["loop"] = {"start": start, "stop": int(rng.integers(start + 1, n + 1)), "times": int(rng.integers(1, 4))}
+    if rng.random() < 0.7:
+        cfg["logit_softcap"] = pick(5.0, 30.0, 50.0)
+    return cfg

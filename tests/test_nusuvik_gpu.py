@@ -79,6 +79,24 @@ def test_schedules_match_the_plain_implementation(models, name, dt, kind):
     check_rows(out, ref, dt, f"{name} {kind}")
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Sizes, order of layers, loop, routers and constants drawn from a seed: a mixed schedule on few pages, both dtypes."""
+    cfg = cases.random_config(seed)
+    w32 = cases.draw_weights(cfg, 100 + seed)
+    reqs = helpers.random_requests(cfg["vocab"], [3, 40, 18, 75, 1, 29], 200 + seed)
+    page = (4, 8, 16, 32)[seed % 4]
+    for dt in ("float32", "bfloat16"):
+        d = cases.write_model(tmp_path / dt, cfg, w32, DT[dt])
+        w = cases.stored(w32, DT[dt])
+        ref = {r: plain.forward(t, w, cfg) for r, t in reqs.items()}
+        steps = schedules.mixed(reqs, seed=seed)
+        eng = _engine(d, dt, page, schedules.max_live_tokens(reqs, steps, page))
+        out = schedules.run(eng, reqs, steps)
+        eng.cache.check_invariants()
+        check_rows(out, ref, dt, f"random configuration {seed}")
+
+
 @pytest.mark.parametrize("name", list(cases.CASES))
 def test_float32_logits_do_not_depend_on_the_schedule(models, name):
     cfg, page, _ = cases.CASES[name]
