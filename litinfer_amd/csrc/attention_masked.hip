@@ -1068,13 +1068,34 @@ extern "C" int li_masked_attention_single(const float* q, int q_token_stride, in
 // thread owns an output and reads its matrix row once for all the tokens.  Sums are float32, in the order of k.
 #define HL_TOK 8
 
+// Behind a head's n_in inputs may lie `n` more columns that are not multiplied but ROTATED by the token's angles
+// (cos, sin [T, n / 2]) and written behind the head's n_out outputs: pairs of neighbouring columns, or (split)
+// column i with column i + n / 2.
+struct HeadTail { int n; int split; const float* cosv; const float* sinv; };
+
+template <typename TX, typename TO>
+__device__ __forceinline__ void head_tail_rotate(const TX* __restrict__ src, TO* __restrict__ dst, int t, int i, const HeadTail& tail) {
+    const int half = tail.n / 2, a = tail.split ? i : 2 * i, b = tail.split ? i + half : 2 * i + 1;
+    const float c = tail.cosv[(size_t)t * half + i], sn = tail.sinv[(size_t)t * half + i];
+    const float u = load_as_float(src + a), v = load_as_float(src + b);
+    store_from_float(dst + a, fmaf(u, c, -__fmul_rn(v, sn)));
+    store_from_float(dst + b, fmaf(v, c, __fmul_rn(u, sn)));
+}
+
 template <typename TX, typename TM, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(
     const TX* __restrict__ x, long x_token_stride, int x_head_stride, const TM* __restrict__ m, TO* __restrict__ out,
-    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride) {
+    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride,
+    HeadTail tail) {
     extern __shared__ float xs[];                    // [HL_TOK][n_in]
     const int h = blockIdx.y, t0 = blockIdx.x * HL_TOK;
     const int nt = (T_ - t0 < HL_TOK) ? T_ - t0 : HL_TOK;
+    if (tail.n > 0 && blockIdx.z == 0)
+        for (int u = threadIdx.x; u < nt * (tail.n / 2); u += 256) {
+            const int tt = u / (tail.n / 2), i = u % (tail.n / 2);
+            head_tail_rotate(x + (size_t)(t0 + tt) * x_token_stride + (size_t)h * x_head_stride + n_in,
+                             out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + n_out, t0 + tt, i, tail);
+        }
     for (int i = threadIdx.x; i < HL_TOK * n_in; i += 256) {
         const int tt = i / n_in, k = i % n_in;
         xs[i] = tt < nt ? load_as_float(x + (size_t)(t0 + tt) * x_token_stride + (size_t)h * x_head_stride + k) : 0.f;
@@ -1132,9 +1153,18 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
 template <typename TX, typename TO>
 __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
     const TX* __restrict__ x, long x_token_stride, int x_head_stride, const bf16_t* __restrict__ m, TO* __restrict__ out,
-    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride) {
+    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in, const float* __restrict__ gate, long gate_stride,
+    HeadTail tail) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h2 = lane >> 5;
     const int head = blockIdx.y, t0 = blockIdx.x * 32;
+    if (tail.n > 0 && blockIdx.z == 0) {
+        const int nt = (T_ - t0 < 32) ? T_ - t0 : 32;
+        for (int u = threadIdx.x; u < nt * (tail.n / 2); u += 256) {
+            const int tt = u / (tail.n / 2), i = u % (tail.n / 2);
+            head_tail_rotate(x + (size_t)(t0 + tt) * x_token_stride + (size_t)head * x_head_stride + n_in,
+                             out + (size_t)(t0 + tt) * o_token_stride + (size_t)head * o_head_stride + n_out, t0 + tt, i, tail);
+        }
+    }
     const int j0 = (blockIdx.z * 4 + w) * 32;
     if (j0 >= n_out) return;
     const int tok = t0 + ql < T_ ? t0 + ql : T_ - 1;
@@ -1178,28 +1208,31 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
 
 template <typename TX, typename TO>
 static bool headwise_mfma(const void* x, long xts, int xhs, const void* m, void* out, long ots, int ohs, int T_, int nh,
-                          int n_out, int n_in, const float* gate, long gate_stride, hipStream_t stream) {
+                          int n_out, int n_in, const float* gate, long gate_stride, HeadTail tail, hipStream_t stream) {
     const int ex = 16 / (int)sizeof(TX) / 2 * 2, eo = 4;       // elements that the 16-byte (32-byte) loads and the stores must start on
     if (T_ < 16 || n_in % 16 || n_out % 32 || xts % ex || xhs % ex || ots % eo || ohs % eo ||
         (uintptr_t)x % 16 || (uintptr_t)m % 16 || (uintptr_t)out % 16)
         return false;
     const dim3 grid((T_ + 31) / 32, nh, (n_out + 127) / 128);
     headwise_linear_mfma_kernel<TX, TO><<<grid, 256, 0, stream>>>((const TX*)x, xts, xhs, (const bf16_t*)m, (TO*)out, ots, ohs,
-                                                                  T_, n_out, n_in, gate, gate_stride);
+                                                                  T_, n_out, n_in, gate, gate_stride, tail);
     return true;
 }
 
 extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_stride, int x_head_stride, const void* m, int m_dtype,
                                   void* out, int out_dtype, long o_token_stride, int o_head_stride, int T_, int nh, int n_out,
-                                  int n_in, const float* gate, long gate_stride, hipStream_t stream) {
+                                  int n_in, const float* gate, long gate_stride, int tail_n, int tail_split, const float* cosv,
+                                  const float* sinv, hipStream_t stream) {
     if (T_ <= 0 || nh <= 0 || nh > 65535 || n_out <= 0 || n_in <= 0 || n_in > 2048 || (gate && gate_stride < nh)) return LI_ERR_SIZE;
+    if (tail_n < 0 || (tail_n & 1) || (tail_n > 0 && (!cosv || !sinv || o_head_stride < n_out + tail_n))) return LI_ERR_SIZE;
+    const HeadTail tail{tail_n, tail_split, cosv, sinv};
     // many tokens against bfloat16 matrices of even sizes: the matrix cores
     if (m_dtype == LI_BF16) {
         bool took = false;
-        if (x_dtype == LI_F32 && out_dtype == LI_F32) took = headwise_mfma<float, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
-        else if (x_dtype == LI_F32 && out_dtype == LI_BF16) took = headwise_mfma<float, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
-        else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) took = headwise_mfma<bf16_t, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
-        else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, stream);
+        if (x_dtype == LI_F32 && out_dtype == LI_F32) took = headwise_mfma<float, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, tail, stream);
+        else if (x_dtype == LI_F32 && out_dtype == LI_BF16) took = headwise_mfma<float, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, tail, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) took = headwise_mfma<bf16_t, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, tail, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, gate, gate_stride, tail, stream);
         if (took) return li_launch_status();
     }
     const int zs = (n_out + 63) / 64;
@@ -1210,10 +1243,10 @@ extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_strid
         constexpr int E = 16 / sizeof(TM);                                                                                 \
         if (n_in % E == 0 && ((uintptr_t)m % 16) == 0)                                                                     \
             headwise_linear_kernel<TX, TM, TO, true><<<grid, 256, lds, stream>>>(                                          \
-                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride); \
+                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride, tail); \
         else                                                                                                               \
             headwise_linear_kernel<TX, TM, TO, false><<<grid, 256, lds, stream>>>(                                         \
-                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride); \
+                (const TX*)x, x_token_stride, x_head_stride, (const TM*)m, (TO*)out, o_token_stride, o_head_stride, T_, n_out, n_in, gate, gate_stride, tail); \
         return li_launch_status();                                                                                         \
     }
     if (x_dtype == LI_F32 && m_dtype == LI_F32 && out_dtype == LI_F32) HL_GO(float, float, float)

@@ -69,7 +69,7 @@ _SIGNATURES = {
         "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L, P, I, I],
-        "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, P, L],
+        "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, P, L, I, I, P, P],
     },
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
@@ -743,12 +743,22 @@ def masked_tiles_take(dk: int, dv: int) -> bool:
 
 
 def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m: torch.Tensor, out: torch.Tensor,
-                    o_token_stride: int, o_head_stride: int, tokens: int, gate: Optional[torch.Tensor] = None) -> None:
+                    o_token_stride: int, o_head_stride: int, tokens: int, gate: Optional[torch.Tensor] = None,
+                    rotate_tail=None) -> None:
     """out[t, h, j] = sum_k m[h, j, k] * x[t, h, k] for m [heads, n_out, n_in]; head h of token t starts at
     t * token_stride + h * head_stride in x (n_in values) and in out (n_out values).  With `gate` (float32 rows
-    [tokens, heads], a view of columns is fine) head h's outputs of token t are multiplied by sigmoid(gate[t, h])."""
+    [tokens, heads], a view of columns is fine) head h's outputs of token t are multiplied by sigmoid(gate[t, h]).
+    With `rotate_tail` = (n, cos, sin, half_split) the n columns behind a head's inputs are rotated by the token's
+    angles (cos, sin [tokens, n / 2]) and written behind the head's outputs."""
     _gpu(x, m, out, gate)
     nh, n_out, n_in = m.shape
+    tn, tcos, tsin, tsplit = rotate_tail if rotate_tail is not None else (0, None, None, False)
+    if tn:
+        _gpu(tcos, tsin)
+        _check_tables("headwise_linear", tokens, tn, tcos, tsin, None)
+        _chk(tn % 2 == 0 and x_head_stride >= n_in + tn and o_head_stride >= n_out + tn
+             and x.numel() >= (tokens - 1) * x_token_stride + (nh - 1) * x_head_stride + n_in + tn
+             and out.numel() >= (tokens - 1) * o_token_stride + (nh - 1) * o_head_stride + n_out + tn, "headwise_linear: the rotated tail")
     _chk(gate is None or (_rows_ok(gate) and gate.dtype is torch.float32 and gate.shape == (tokens, nh)), "headwise_linear: gate")
     _chk(m.is_contiguous() and m.dtype in _DT and x.dtype in _DT and out.dtype in _DT and x.is_contiguous()
          and out.is_contiguous(), "headwise_linear: operands")
@@ -760,7 +770,8 @@ def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m:
     if tokens:
         _run("attention_masked", "li_headwise_linear", x.data_ptr(), _DT[x.dtype], int(x_token_stride), int(x_head_stride),
              m.data_ptr(), _DT[m.dtype], out.data_ptr(), _DT[out.dtype], int(o_token_stride), int(o_head_stride),
-             tokens, nh, n_out, n_in, 0 if gate is None else gate.data_ptr(), 0 if gate is None else gate.stride(0))
+             tokens, nh, n_out, n_in, 0 if gate is None else gate.data_ptr(), 0 if gate is None else gate.stride(0),
+             int(tn), int(bool(tsplit)), tcos.data_ptr() if tn else 0, tsin.data_ptr() if tn else 0)
 
 
 # ---------------------------------------------------------------------- gemm

@@ -197,19 +197,20 @@ class LatentAttention(Mixer):
         down = qd[:, n_first:n_first + rank + dr]
         if self.q_rank:
             # the norm of the queries' latent, the norm of the keys' latent, the rotation of the shared key part and the
-            # page write: one kernel; then the queries themselves, and the rotation of their rotated parts
+            # page write: one kernel; then the queries themselves, whose rotated parts the per-head product rotates
+            # on their way behind its outputs
             cq = ctx.ws.buffer("latent.cq", (t, self.q_rank), self.rt.dtype)
             ops.latent_norm_pairs_store(None, 0, dn, dr, rank, self.wc, self.eps, cos, sin, slots, rows if cache.owned else None,
                                         None, down=down, half_split=self.half_split, q_latent=qd[:, :self.q_rank], wq=self.wq, cq=cq)
             q = ctx.ws.buffer("latent.q32", (t, self.n_q), torch.float32)
             self.q_up(cq, q, ws=ctx.ws)
-            ops.latent_norm_pairs_store(q, nh, dn, dr, rank, self.wc, self.eps, cos, sin, None, None, qfull, down=down,
-                                        half_split=self.half_split)
+            ops.headwise_linear(q, q.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t,
+                                rotate_tail=(dr, cos, sin, self.half_split))
         else:
             q = qd
             ops.latent_norm_pairs_store(qd, nh, dn, dr, rank, self.wc, self.eps, cos, sin, slots, rows if cache.owned else None,
                                         qfull, half_split=self.half_split)
-        ops.headwise_linear(q, q.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
+            ops.headwise_linear(q, q.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
         summed = ctx.ws.buffer("latent.summed", (t, nh * rank), self.rt.dtype)
         ops.masked_attention(qfull, nh * (rank + dr), rank + dr, summed, rows, rows, ctx.attention_meta(cache.group),
                              nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale,

@@ -375,6 +375,36 @@ def test_layer_norm_gelu_rows_side_by_side_and_gated_products():
         assert np.abs(out.float().cpu().numpy().reshape(T, nh, n_out) - ref).max() < (1e-5 if dt is torch.float32 else 2e-2) * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("T,nh,n_out,n_in,tail,mdt", [(5, 3, 40, 24, 8, torch.float32), (70, 4, 64, 32, 64, torch.bfloat16),
+                                                      (33, 2, 20, 48, 2, torch.bfloat16), (200, 8, 192, 64, 32, torch.bfloat16)])
+def test_per_head_product_that_rotates_the_columns_behind_its_inputs(split, T, nh, n_out, n_in, tail, mdt):
+    """Queries into the latent space: a head's plain columns are multiplied, its rotated columns behind them are
+    rotated and written behind the outputs, on both paths of the kernel."""
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(T)
+    f32 = lambda a: torch.tensor(a, dtype=torch.float32, device=DEV)
+    m = torch.tensor(rng.normal(size=(nh, n_out, n_in)), dtype=torch.float32).to(mdt)
+    x = rng.normal(size=(T, nh, n_in + tail))
+    pos = rng.integers(0, 900, T)
+    ang = pos[:, None] * np.array([70.0 ** (-2.0 * i / tail) for i in range(tail // 2)])
+    out = torch.full((T, nh, n_out + tail), 7.0, device=DEV)
+    ops.headwise_linear(f32(x.reshape(T, -1)), nh * (n_in + tail), n_in + tail, m.to(DEV), out, nh * (n_out + tail), n_out + tail, T,
+                        rotate_tail=(tail, f32(np.cos(ang)), f32(np.sin(ang)), split))
+    got = out.cpu().numpy()
+    ref = np.einsum("hjk,thk->thj", m.double().numpy(), x[:, :, :n_in])
+    assert np.abs(got[:, :, :n_out] - ref).max() < (1e-5 if mdt is torch.float32 else 2e-2) * np.abs(ref).max()
+    for h in range(nh):
+        r = x[:, h, n_in:]
+        if split:
+            want = plain.rotate_half(r, pos, 70.0, tail)
+        else:
+            want = np.empty_like(r)
+            want[:, 0::2] = r[:, 0::2] * np.cos(ang) - r[:, 1::2] * np.sin(ang)
+            want[:, 1::2] = r[:, 1::2] * np.cos(ang) + r[:, 0::2] * np.sin(ang)
+        assert np.abs(got[:, h, n_out:] - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,dn,dr,rank,q_rank", [(3, 24, 8, 40, 56), (1, 48, 16, 64, 32), (4, 32, 64, 64, 96), (5, 8, 24, 8, 16)])
 def test_norms_rotation_and_page_write_of_the_latent_mixer(dt, nh, dn, dr, rank, q_rank):
