@@ -1100,6 +1100,10 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
         const int tt = i / n_in, k = i % n_in;
         xs[i] = tt < nt ? load_as_float(x + (size_t)(t0 + tt) * x_token_stride + (size_t)h * x_head_stride + k) : 0.f;
     }
+    // the heads' gates are asked for before the products, so that they have arrived when the outputs are ready
+    float gf[HL_TOK];
+#pragma unroll
+    for (int tt = 0; tt < HL_TOK; ++tt) gf[tt] = gate ? gate[(size_t)(t0 + (tt < nt ? tt : 0)) * gate_stride + h] : 0.f;
     __syncthreads();
     // four neighbouring threads share an output: each takes every fourth piece of the matrix row
     constexpr int E = VEC ? 16 / (int)sizeof(TM) : 1;
@@ -1140,7 +1144,7 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
         }
         if (on && part == 0)
             for (int tt = 0; tt < nt; ++tt) {
-                const float f = gate ? 1.0f / (1.0f + expf(-gate[(size_t)(t0 + tt) * gate_stride + h])) : 1.0f;
+                const float f = gate ? 1.0f / (1.0f + expf(-gf[tt])) : 1.0f;
                 store_from_float(out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + j, acc[tt] * f);
             }
     }
