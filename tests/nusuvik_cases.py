@@ -117,7 +117,7 @@ def random_config(seed):
         heads, dim, rot = pick(1, 2, 3, 4, 6, 8, 16), pick(8, 16, 24, 32, 64, 128), pick(2, 8, 16, 32, 64)
         return dict(heads=heads, dim=dim, rot_dim=rot, vdim=pick(8, 16, 32, 48, 64, 128), kv_rank=pick(8, 24, 32, 64, 96, 128),
                     q_rank=pick(8, 16, 48, 64, 128, 192), scale=float(rng.uniform(0.5, 1.5)) / np.sqrt(dim + rot),
-                    base=pick(100.0, 10000.0, 1000000.0))
+                    base=pick(100.0, 10000.0, 500000.0))
     shared = mixer()
     layers = []
     for i in range(n):
@@ -135,12 +135,12 @@ def random_config(seed):
             mlp = None
         kinds.append(kind)
         layers.append(latent_layer(m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"], m["scale"], mlp, m["base"]))
-    cfg = {"architecture": "Nusuvik", "vocab": pick(61, 200, 448, 515), "width": width, "norm": {"eps": pick(1e-6, 1e-5, 1e-3)}, "layers": layers}
+    cfg = {"architecture": "Nusuvik", "vocab": pick(61, 200, 450, 515), "width": width, "norm": {"eps": pick(1e-6, 1e-5, 1e-3)}, "layers": layers}
     if rng.random() < 0.8:
-        cfg["embedding"] = {"bigram": {"buckets": pick(7, 509, 4099), "mul_prev": pick(1, 31, 65537), "mul_cur": pick(1, 7, 1009)}}
+        cfg["embedding"] = {"bigram": {"buckets": pick(7, 521, 4099), "mul_prev": pick(1, 37, 65537), "mul_cur": pick(1, 11, 1009)}}
     if rng.random() < 0.8:
         start = int(rng.integers(0, n))
         cfg["loop"] = {"start": start, "stop": int(rng.integers(start + 1, n + 1)), "times": int(rng.integers(1, 4))}
     if rng.random() < 0.7:
-        cfg["logit_softcap"] = pick(5.0, 30.0, 50.0)
+        cfg["logit_softcap"] = pick(5.0, 25.0, 50.0)
     return cfg
