@@ -557,3 +557,31 @@ def test_dense_feed_forward_with_biases(dt):
         part.forward(h.to(DEV), ResidualStream(x, ws), SimpleNamespace(ws=ws))
         ref = plain.dense_mlp(h.double().numpy(), {n: a.double().numpy() for n, a in wt.items()}, "")
         assert np.abs(x.cpu().numpy() - x0 - ref).max() < (1e-5 if dt == "float32" else 2e-2) * np.abs(ref).max()
+
+
+# ------------------------------------------------------------------------------- as a user runs it, in a subprocess
+def test_generate_through_the_command_line(models):
+    from test_cli import cli, last_json
+    cfg, page, seed = cases.CASES["D"]
+    d, reqs, _ = models[("D", "float32")]
+    w = cases.stored(cases.draw_weights(cfg, seed), torch.float32)
+    prompt = reqs["r1"]
+    out = last_json(cli("generate", "--model", d, "--test", "--max_steps", 10, "--dtype", "float32", "--page-size", page,
+                        "--chunk-size", 6, "--prompt-ids", ",".join(map(str, prompt))).stdout)
+    assert len(out["tokens"]) == 10
+    seq = list(prompt)
+    for t in out["tokens"]:
+        logits = plain.forward(seq, w, cfg)[-1]
+        assert logits.max() - logits[t] < 1e-4 * np.abs(logits).max(), (len(seq), t)
+        seq.append(int(t))
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_trace_replay_in_a_subprocess(models, tmp_path, dt):
+    from test_trace_run_gpu import replay
+    d, reqs, ref = models[("C", dt)]
+    some = {r: reqs[r] for r in ("r0", "r1", "r3", "r5", "r7", "r8")}
+    for kind in ("chunks", "mixed"):
+        steps = getattr(schedules, kind)(some)
+        out = replay(d, dt, some, steps, tmp_path / f"out_{kind}", schedules.max_live_tokens(some, steps))
+        check_rows(out, {r: ref[r] for r in some}, dt, f"replay {kind}")
