@@ -20,6 +20,10 @@ from .nusuvik import NusuvikConfig, nusuvik_model_spec
 
 register_architecture("Nusuvik", NusuvikConfig.from_dict, nusuvik_model_spec, aliases=("nusuvik",))
 
-__all__ = ["NusuvikConfig", "nusuvik_model_spec", "TovasunConfig", "tovasun_model_spec", "SogenexConfig", "sogenex_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
+from .kufolorn import KufolornConfig, kufolorn_model_spec
+
+register_architecture("Kufolorn", KufolornConfig.from_dict, kufolorn_model_spec, aliases=("kufolorn",))
+
+__all__ = ["KufolornConfig", "kufolorn_model_spec", "NusuvikConfig", "nusuvik_model_spec", "TovasunConfig", "tovasun_model_spec", "SogenexConfig", "sogenex_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
            "load_config", "lookup", "read_config_json", "register_architecture",
            "registered_architectures", "ConfigError", "Qwen2Config", "qwen2_model_spec"]

@@ -19,6 +19,17 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// What a (token, head)'s sums of values are multiplied by at the end: one over the sum of the weights, to which a
+// softmax with a SINK adds exp(sink[head] - maximum) (a term of the denominator that has no key and no value), and,
+// where the heads have gates, times sigmoid(gate[token, head]).
+__device__ __forceinline__ float finish_factor(float l, float m, const float* __restrict__ sink, const float* __restrict__ gate,
+                                               long gate_stride, int t, int head) {
+    if (sink && l != 0.f) l += expf(sink[head] - m);
+    float f = l != 0.f ? 1.0f / l : 0.f;
+    if (gate) f *= 1.0f / (1.0f + expf(-gate[(size_t)t * gate_stride + head]));
+    return f;
+}
+
 // The general kernel (any sizes, both dtypes): a block of NW waves per (token, query head); wave w takes the
 // rounds w, w + NW, ... of 64 visible keys.  In a round a lane takes one key for the scores (its row read in
 // 16-byte pieces where the rows allow it), then one value column (and every 64th after it) for the sums.  The
@@ -30,7 +41,7 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_wave_kernel(
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
     const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
-    int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale) {
+    int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale, const float* __restrict__ sink, const float* __restrict__ gate, long gate_stride) {
     extern __shared__ float smem[];
     float* qs = smem;                                        // [dk]
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -114,10 +125,11 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_wave_kernel(
     }
     TO* orow = out + ((size_t)t * nh + h) * dv;
     if constexpr (NW == 1) {
+        const float fin = finish_factor(l, m, sink, gate, gate_stride, t, h);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int d = lane + c * LI_WAVE;
-            if (d < dv) store_from_float(orow + d, l != 0.f ? acc[c] / l : 0.f);
+            if (d < dv) store_from_float(orow + d, acc[c] * fin);
         }
     } else {
         float* mine = join + (size_t)w * (dv + 2);
@@ -138,11 +150,12 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_wave_kernel(
             f[x] = (lx == 0.f) ? 0.f : expf(mx - mm);
             ll += lx * f[x];
         }
+        const float fin = finish_factor(ll, mm, sink, gate, gate_stride, t, h);
         for (int d = threadIdx.x; d < dv; d += 64 * NW) {
             float a = 0.f;
 #pragma unroll
             for (int x = 0; x < NW; ++x) a += join[(size_t)x * (dv + 2) + d] * f[x];
-            store_from_float(orow + d, ll != 0.f ? a / ll : 0.f);
+            store_from_float(orow + d, a * fin);
         }
     }
 }
@@ -152,14 +165,14 @@ static int launch_masked(const float* q, int qts, int qhs, void* out, const void
                          const int* block_table, int max_blocks, const int* token_list, int n_tokens, const int* seg_of_token,
                          const int* q_start, const int* q_len,
                          const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
-                         int keep_first, float softcap, float scale, int waves, hipStream_t stream) {
+                         int keep_first, float softcap, float scale, const float* sink, const float* gate, long gate_stride, int waves, hipStream_t stream) {
     const dim3 grid(n_tokens, nh);
     constexpr int E = 16 / sizeof(T);
     const bool vec = dk % E == 0 && k_row % E == 0 && ((uintptr_t)kc % 16) == 0;
 #define MA_GO(V, NW)                                                                                                         \
     masked_attention_wave_kernel<T, TO, NC, V, NW><<<grid, 64 * NW, (size_t)(dk + NW * 128 + NW * (dv + 2)) * 4, stream>>>(  \
         q, qts, qhs, (TO*)out, (const T*)kc, (const T*)vc, k_row, v_row, block_table, max_blocks, token_list, seg_of_token,  \
-        q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap, scale)
+        q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap, scale, sink, gate, gate_stride)
     if (waves >= 8) { if (vec) MA_GO(true, 8); else MA_GO(false, 8); }
     else if (waves >= 4) { if (vec) MA_GO(true, 4); else MA_GO(false, 4); }
     else { if (vec) MA_GO(true, 1); else MA_GO(false, 1); }
@@ -177,7 +190,7 @@ extern "C" int li_masked_attention(const float* q, int q_token_stride, int q_hea
                                    const int* block_table, int max_blocks, const int* token_list, int n_tokens,
                                    const int* seg_of_token, const int* q_start,
                                    const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv,
-                                   int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
+                                   int page_size, int num_pages, int window, int keep_first, float softcap, float scale, const float* sink, const float* gate, long gate_stride,
                                    int waves, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dv <= 0 || dk > k_row || dv > v_row || page_size <= 0 ||
         window < 0 || keep_first < 0 || max_blocks <= 0 || nh > 65535 || dk > 4096 || dv > 64 * MA_MAX_CHUNKS)
@@ -185,7 +198,7 @@ extern "C" int li_masked_attention(const float* q, int q_token_stride, int q_hea
     const int nc = (dv + 63) / 64;
 #define MA_ARGS q, q_token_stride, q_head_stride, out, kc, vc, k_row, v_row, block_table, max_blocks, token_list, n_tokens,  \
                 seg_of_token, q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap,   \
-                scale, waves, stream
+                scale, sink, gate, gate_stride, waves, stream
 #define MA_PICK(T, TO)                                                                  \
     {                                                                                   \
         if (nc <= 1) return launch_masked<T, TO, 1>(MA_ARGS);                           \
@@ -233,7 +246,7 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
-    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
+    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale, const float* __restrict__ sink, const float* __restrict__ gate, long gate_stride,
     int nsplit, float* __restrict__ parts) {
     constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
     constexpr int NT = NW * 64;
@@ -437,7 +450,7 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
         if (h == 0) { part[DV] = m; part[DV + 1] = l; }
         return;
     }
-    const float inv = l != 0.f ? 1.0f / l : 0.f;
+    const float inv = finish_factor(l, m, sink, gate, gate_stride, t0 + ql, head);
     bf16_t* orow = out + ((size_t)(t0 + ql) * nh + head) * DV;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -450,7 +463,8 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
 }
 
 __global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
-                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, int by_token = 0);
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, const float* __restrict__ sink,
+                                             const float* __restrict__ gate, long gate_stride, int by_token = 0);
 
 // ------------------------------------------------------------------------------------------- single tokens, MFMA
 // Decoding where a kv head serves many query heads (a compressed cache serves ALL of them): the same transposed
@@ -463,7 +477,7 @@ __global__ __launch_bounds__(64) void masked_attention_heads_kernel(
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
     const int* __restrict__ seg_of_token, const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
-    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
+    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale, const float* __restrict__ sink, const float* __restrict__ gate, long gate_stride,
     int nsplit, float* __restrict__ parts) {
     constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
     constexpr int NT = 64;
@@ -639,7 +653,7 @@ __global__ __launch_bounds__(64) void masked_attention_heads_kernel(
     l += __shfl_xor(l, 32, LI_WAVE);
     if (!has) return;
     if (nsplit == 1) {
-        const float inv = l != 0.f ? 1.0f / l : 0.f;
+        const float inv = finish_factor(l, m, sink, gate, gate_stride, t, head);
         bf16_t* orow = out + ((size_t)t * nh + head) * DV;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -674,7 +688,7 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
                                          const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
                                          const int* tiles, int num_tiles, const int* q_start, const int* q_len,
                                          const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages,
-                                         int window, int keep_first, float softcap, float scale, int nsplit, float* parts,
+                                         int window, int keep_first, float softcap, float scale, const float* sink, const float* gate, long gate_stride, int nsplit, float* parts,
                                          long parts_floats, const int* multi_tokens, int num_multi, int num_tokens,
                                          hipStream_t stream) {
     if (num_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
@@ -693,15 +707,15 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
         if (nw == 8)                                                                                                       \
             masked_attention_tile_kernel<K / 16, V / 32, 8><<<grid, 512, 0, stream>>>(                                     \
                 q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
-                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, sink, gate, gate_stride, \
                 nsplit, parts);                                                                                            \
         else                                                                                                               \
             masked_attention_tile_kernel<K / 16, V / 32, 4><<<grid, 256, 0, stream>>>(                                     \
                 q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
-                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, sink, gate, gate_stride, \
                 nsplit, parts);                                                                                            \
         if (nsplit > 1)                                                                                                    \
-            masked_attention_join_kernel<<<dim3(num_multi, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, multi_tokens, nh, dv, nsplit, 1); \
+            masked_attention_join_kernel<<<dim3(num_multi, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, multi_tokens, nh, dv, nsplit, sink, gate, gate_stride, 1); \
         return li_launch_status();                                                                                         \
     }
     MT_GO(64, 64) MT_GO(128, 128) MT_GO(128, 64) MT_GO(64, 128) MT_GO(96, 64) MT_GO(160, 128) MT_GO(192, 128)
@@ -715,7 +729,7 @@ extern "C" int li_masked_attention_heads(const float* q, int q_token_stride, int
                                          const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
                                          const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
                                          const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size,
-                                         int num_pages, int window, int keep_first, float softcap, float scale, int nsplit,
+                                         int num_pages, int window, int keep_first, float softcap, float scale, const float* sink, const float* gate, long gate_stride, int nsplit,
                                          float* parts, long parts_floats, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
         window < 0 || keep_first < 0 || max_blocks <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 || q_head_stride % 4 ||
@@ -729,9 +743,9 @@ extern "C" int li_masked_attention_heads(const float* q, int q_token_stride, int
         masked_attention_heads_kernel<K / 16, V / 32><<<grid, 64, 0, stream>>>(                                            \
             q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
             max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, \
-            softcap, scale, nsplit, parts);                                                                                \
+            softcap, scale, sink, gate, gate_stride, nsplit, parts);                                                                                \
         if (nsplit > 1)                                                                                                    \
-            masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit); \
+            masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit, sink, gate, gate_stride); \
         return li_launch_status();                                                                                         \
     }
     MH_GO(64, 64) MH_GO(128, 128) MH_GO(128, 64) MH_GO(64, 128) MH_GO(96, 64) MH_GO(160, 128) MH_GO(192, 128)
@@ -775,7 +789,7 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
     const int* __restrict__ seg_of_token, const int* __restrict__ q_start, const int* __restrict__ q_len,
     const int* __restrict__ ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
-    int keep_first, float softcap, float scale, int tab_cap, int pshift, int nsplit, float* __restrict__ parts) {
+    int keep_first, float softcap, float scale, const float* __restrict__ sink, const float* __restrict__ gate, long gate_stride, int tab_cap, int pshift, int nsplit, float* __restrict__ parts) {
     extern __shared__ float join[];                 // [4 waves][RH][dv + 2], then tab_cap table entries
     int* tab = (int*)(join + (size_t)4 * RH * (dv + 2));
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, g = lane >> 3, j = lane & 7;
@@ -967,7 +981,7 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
         }
         const int head = kvh * rep + hfirst + hh;
         if (nsplit == 1) {
-            out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
+            out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(a * finish_factor(ll, mm, sink, gate, gate_stride, t, head));
         } else {                                    // this split's sums, maximum and sum of weights: joined by the kernel behind
             float* part = parts + (((size_t)blockIdx.x * nh + head) * nsplit + sp) * (dv + 2);
             part[d] = a;
@@ -979,7 +993,8 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
 // joins the splits of every (token, head) in split order: a block a (token, head)
 // (the parts of a token lie at its place in the list, or, with by_token, at its own number)
 __global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
-                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, int by_token) {
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, const float* __restrict__ sink,
+                                             const float* __restrict__ gate, long gate_stride, int by_token) {
     const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, head = blockIdx.y;
     const float* base = parts + ((size_t)(by_token ? t : (int)blockIdx.x) * nh + head) * nsplit * (dv + 2);
     float mm = -INFINITY;
@@ -992,7 +1007,7 @@ __global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf
             a += r[d] * f;
             ll += r[dv + 1] * f;
         }
-        out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
+        out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(a * finish_factor(ll, mm, sink, gate, gate_stride, t, head));
     }
 }
 
@@ -1014,7 +1029,7 @@ extern "C" int li_masked_attention_single(const float* q, int q_token_stride, in
                                           const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
                                           const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
                                           const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size,
-                                          int num_pages, int window, int keep_first, float softcap, float scale,
+                                          int num_pages, int window, int keep_first, float softcap, float scale, const float* sink, const float* gate, long gate_stride,
                                           int nsplit, float* parts, long parts_floats, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
         window < 0 || keep_first < 0 || max_blocks <= 0 || num_pages <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 ||
@@ -1035,10 +1050,10 @@ extern "C" int li_masked_attention_single(const float* q, int q_token_stride, in
     masked_attention_single_kernel<K, V, R, UU><<<grid, 256, lds, stream>>>(                                                \
         q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table,    \
         max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window,       \
-        keep_first, softcap, scale, tab_cap, pshift, nsplit, parts)
+        keep_first, softcap, scale, sink, gate, gate_stride, tab_cap, pshift, nsplit, parts)
 #define MS_JOIN                                                                                                             \
     if (nsplit > 1)                                                                                                         \
-        masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit);
+        masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit, sink, gate, gate_stride);
 #define MS_SMALL(K, V)                                                                                                      \
     if (npk == K && npv == V) {                                                                                             \
         if (rh == 4) MS_GO(K, V, 4, 4); else if (rh == 2) MS_GO(K, V, 2, 4); else MS_GO(K, V, 1, 4);                        \

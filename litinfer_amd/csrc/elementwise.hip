@@ -188,6 +188,37 @@ extern "C" int li_swiglu(const void* gu, void* out, int dtype, int T, int I, hip
     return li_launch_status();
 }
 
+// out[t, i] = act(gate) * up with gate = gu[t, i], up = gu[t, I + i]; act 0: z / (1 + exp(-z)),
+// act 1: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).  Arithmetic in float32.
+template <typename TI, typename TO>
+__global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int I, int act) {
+    const TI* g = gu + (size_t)blockIdx.y * 2 * I;
+    TO* o = out + (size_t)blockIdx.y * I;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < I) {
+        const float gv = load_as_float(g + i), uv = load_as_float(g + I + i);
+        const float a = act == 1 ? 0.5f * gv * (1.0f + tanhf(0.7978845608028654f * (gv + 0.044715f * gv * gv * gv)))
+                                 : gv / (1.0f + expf(-gv));
+        store_from_float(o + i, a * uv);
+    }
+}
+
+extern "C" int li_gated_act(const void* gu, int in_dtype, void* out, int out_dtype, int T, int I, int act, hipStream_t stream) {
+    if (T <= 0 || I <= 0 || T > 65535 * 32 || act < 0 || act > 1) return LI_ERR_SIZE;
+    for (int t0 = 0; t0 < T; t0 += 65535) {
+        const int rows = (T - t0 < 65535) ? T - t0 : 65535;
+        dim3 grid((I + 255) / 256, rows);
+        if (in_dtype == LI_F32 && out_dtype == LI_F32)
+            gated_act_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)gu + (size_t)t0 * 2 * I, (float*)out + (size_t)t0 * I, I, act);
+        else if (in_dtype == LI_F32 && out_dtype == LI_BF16)
+            gated_act_kernel<float, bf16_t><<<grid, 256, 0, stream>>>((const float*)gu + (size_t)t0 * 2 * I, (bf16_t*)out + (size_t)t0 * I, I, act);
+        else if (in_dtype == LI_BF16 && out_dtype == LI_BF16)
+            gated_act_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu + (size_t)t0 * 2 * I, (bf16_t*)out + (size_t)t0 * I, I, act);
+        else return LI_ERR_DTYPE;
+    }
+    return li_launch_status();
+}
+
 // --------------------------------------------------------------------- rope
 // angle = float(pos) / powf(theta, float(2j) / rotary_dim); cos and sin in float32
 __global__ void rope_table_kernel(const int* __restrict__ pos, float theta, int rotary_dim,
@@ -416,43 +447,51 @@ extern "C" int li_embedding_add(const int* ids, const int* id_src, const int* fe
     return li_launch_status();
 }
 
-// x[t, :] += y[t, :] / sqrt(mean(y^2) + eps) * w, and, where w2 is given, xn[t, :] = the RMS norm
-// of the NEW x with weights w2 and eps2 (the norm through which the stream is read next): one block a row.
+// x[t, :] += b / sqrt(mean(b^2) + eps) * w for the branch b = y (or, with y2, b = a1 y + a2 y2), and, for whoever
+// reads the stream next, xn[t, :] = the RMS norm of the NEW x with weights w2 and eps2 (next 1) or the new x itself in
+// xn's type (next 2): one block a row.
 template <typename TO, int NT>
-__global__ __launch_bounds__(NT) void rmsnorm_add_kernel(const float* __restrict__ y, const float* __restrict__ w, float eps,
+__global__ __launch_bounds__(NT) void rmsnorm_add_kernel(const float* __restrict__ y, const float* __restrict__ y2, float a1, float a2,
+                                                          const float* __restrict__ w, float eps,
                                                           float* __restrict__ x, const float* __restrict__ w2, float eps2,
-                                                          TO* __restrict__ xn, int H) {
+                                                          TO* __restrict__ xn, int next, int H) {
     __shared__ float red[NT / LI_WAVE];
     const float* yr = y + (size_t)blockIdx.x * H;
+    const float* yr2 = y2 ? y2 + (size_t)blockIdx.x * H : nullptr;
     float* xr = x + (size_t)blockIdx.x * H;
     float ss = 0.f;
-    for (int j = threadIdx.x; j < H; j += NT) { const float v = yr[j]; ss += v * v; }
+    for (int j = threadIdx.x; j < H; j += NT) { const float v = yr2 ? a1 * yr[j] + a2 * yr2[j] : yr[j]; ss += v * v; }
     ss = block_sum<NT>(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)H + eps);
     float s2 = 0.f;
     for (int j = threadIdx.x; j < H; j += NT) {
-        const float v = xr[j] + yr[j] * inv * w[j];
+        const float b = yr2 ? a1 * yr[j] + a2 * yr2[j] : yr[j];
+        const float v = xr[j] + b * inv * w[j];
         xr[j] = v;
         s2 += v * v;
     }
-    if (w2 == nullptr) return;
+    if (next == 0) return;
+    TO* o = xn + (size_t)blockIdx.x * H;
+    if (next == 2) {
+        for (int j = threadIdx.x; j < H; j += NT) store_from_float(o + j, xr[j]);               // (a thread reads back what it wrote)
+        return;
+    }
     s2 = block_sum<NT>(s2, red);
     const float inv2 = 1.0f / sqrtf(s2 / (float)H + eps2);
-    TO* o = xn + (size_t)blockIdx.x * H;
-    for (int j = threadIdx.x; j < H; j += NT) store_from_float(o + j, xr[j] * inv2 * w2[j]);     // (a thread reads back what it wrote)
+    for (int j = threadIdx.x; j < H; j += NT) store_from_float(o + j, xr[j] * inv2 * w2[j]);
 }
 
-extern "C" int li_rmsnorm_add(const float* y, const float* w, float eps, float* x, const float* w2, float eps2,
-                              void* xn, int xn_dtype, int T, int H, hipStream_t stream) {
-    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
-    if (w2 && !xn) return LI_ERR_SIZE;
+extern "C" int li_rmsnorm_add(const float* y, const float* y2, float a1, float a2, const float* w, float eps, float* x,
+                              const float* w2, float eps2, void* xn, int xn_dtype, int next, int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || next < 0 || next > 2) return LI_ERR_SIZE;
+    if ((next && !xn) || (next == 1 && !w2)) return LI_ERR_SIZE;
     const bool wide = T < 256 && H > 1024;
 #define LI_RA(TO)                                                                                             \
     {                                                                                                         \
-        if (wide) rmsnorm_add_kernel<TO, 1024><<<T, 1024, 0, stream>>>(y, w, eps, x, w2, eps2, (TO*)xn, H);   \
-        else rmsnorm_add_kernel<TO, 256><<<T, 256, 0, stream>>>(y, w, eps, x, w2, eps2, (TO*)xn, H);          \
+        if (wide) rmsnorm_add_kernel<TO, 1024><<<T, 1024, 0, stream>>>(y, y2, a1, a2, w, eps, x, w2, eps2, (TO*)xn, next, H);   \
+        else rmsnorm_add_kernel<TO, 256><<<T, 256, 0, stream>>>(y, y2, a1, a2, w, eps, x, w2, eps2, (TO*)xn, next, H);          \
     }
-    if (!w2 || xn_dtype == LI_F32) LI_RA(float)
+    if (!next || xn_dtype == LI_F32) LI_RA(float)
     else if (xn_dtype == LI_BF16) LI_RA(bf16_t)
     else return LI_ERR_DTYPE;
 #undef LI_RA
@@ -568,14 +607,14 @@ extern "C" int li_rope_pairs_apply(void* x, int dtype, int row_stride, int n_hea
 
 // The step between the packed q/k/v projection (float32 rows [q | k | v]) and the attention, for a mixer that
 // norms the WHOLE query projection and the WHOLE key projection (all heads at once, before they are split) and
-// rotates neighbouring pairs: q is normed and rotated in place (it stays float32), k is normed, rotated and
+// rotates pairs of columns (neighbours, or with half_split column i and column i + rotary_dim / 2): q is normed and rotated in place (it stays float32), k is normed, rotated and
 // written to its page slot, v is copied to its page slot.  wq / wk null: no norm.  One block a token.
 template <typename T, int NT>
 __global__ __launch_bounds__(NT) void qk_norm_pairs_store_kernel(
     float* __restrict__ qkv, int row_stride, int nh, int nkv, int dk, int dv, int rotary_dim,
     const float* __restrict__ wq, const float* __restrict__ wk, float eps,
     const float* __restrict__ cosv, const float* __restrict__ sinv, const int* __restrict__ slot_map,
-    T* __restrict__ kc, T* __restrict__ vc, int page_size, int store) {
+    T* __restrict__ kc, T* __restrict__ vc, int page_size, int store, int half_split) {
     __shared__ float red[NT / LI_WAVE];
     const int t = blockIdx.x, half = rotary_dim / 2;
     float* q = qkv + (size_t)t * row_stride;
@@ -601,11 +640,11 @@ __global__ __launch_bounds__(NT) void qk_norm_pairs_store_kernel(
     for (int u = threadIdx.x; u < nh * units; u += NT) {
         const int h = u / units, i = u % units;
         if (i < half) {
-            const int j = h * dk + 2 * i;
-            const float a = wq ? q[j] * inv_q * wq[j] : q[j], b = wq ? q[j + 1] * inv_q * wq[j + 1] : q[j + 1];
+            const int j = h * dk + (half_split ? i : 2 * i), j2 = half_split ? j + half : j + 1;    // the pair's two columns
+            const float a = wq ? q[j] * inv_q * wq[j] : q[j], b = wq ? q[j2] * inv_q * wq[j2] : q[j2];
             float ra, rb;
             rotate_pair(a, b, c[i], sn[i], ra, rb);
-            q[j] = ra; q[j + 1] = rb;
+            q[j] = ra; q[j2] = rb;
         } else if (wq) {
             const int j = h * dk + rotary_dim + (i - half);
             q[j] = q[j] * inv_q * wq[j];
@@ -617,12 +656,13 @@ __global__ __launch_bounds__(NT) void qk_norm_pairs_store_kernel(
         const int h = u / units, i = u % units;
         T* dst = kc + ((size_t)(page * nkv + h) * page_size + off) * dk;
         if (i < half) {
-            const int j = h * dk + 2 * i;
-            const float a = wk ? k[j] * inv_k * wk[j] : k[j], b = wk ? k[j + 1] * inv_k * wk[j + 1] : k[j + 1];
+            const int d1 = half_split ? i : 2 * i, d2 = half_split ? i + half : 2 * i + 1;
+            const int j = h * dk + d1, j2 = h * dk + d2;
+            const float a = wk ? k[j] * inv_k * wk[j] : k[j], b = wk ? k[j2] * inv_k * wk[j2] : k[j2];
             float ra, rb;
             rotate_pair(a, b, c[i], sn[i], ra, rb);
-            store_from_float(dst + 2 * i, ra);
-            store_from_float(dst + 2 * i + 1, rb);
+            store_from_float(dst + d1, ra);
+            store_from_float(dst + d2, rb);
         } else {
             const int d = rotary_dim + (i - half), j = h * dk + d;
             store_from_float(dst + d, wk ? k[j] * inv_k * wk[j] : k[j]);
@@ -637,7 +677,7 @@ __global__ __launch_bounds__(NT) void qk_norm_pairs_store_kernel(
 extern "C" int li_qk_norm_pairs_store(float* qkv, int row_stride, int nh, int nkv, int dk, int dv, int rotary_dim,
                                       const float* wq, const float* wk, float eps, const float* cosv, const float* sinv,
                                       const int* slot_map, void* kc, void* vc, int cache_dtype, int page_size, int store,
-                                      int T, hipStream_t stream) {
+                                      int half_split, int T, hipStream_t stream) {
     if (T <= 0 || nh <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > dk ||
         row_stride < nh * dk + nkv * (dk + dv) || page_size <= 0)
         return LI_ERR_SIZE;
@@ -646,9 +686,9 @@ extern "C" int li_qk_norm_pairs_store(float* qkv, int row_stride, int nh, int nk
 #define LI_QK(TC)                                                                                                            \
     {                                                                                                                        \
         if (wide) qk_norm_pairs_store_kernel<TC, 1024><<<T, 1024, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps, \
-                                                                              cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store); \
+                                                                              cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store, half_split); \
         else qk_norm_pairs_store_kernel<TC, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,  \
-                                                                        cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store);  \
+                                                                        cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store, half_split);  \
     }
     if (cache_dtype == LI_F32) LI_QK(float)
     else if (cache_dtype == LI_BF16) LI_QK(bf16_t)

@@ -14,7 +14,9 @@
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
 // largest (the lower index wins a tie), weights = softmax over the chosen logits.  gate[t] = sigmoid(wg . x).
 // mode 1: scores are sigmoid(logit), the choice goes by score + corr[e] inside the best groups of neighbouring
-// experts, the weights are the chosen scores over their sum.
+// experts, the weights are the chosen scores over their sum.  mode 2: the same with scores = softmax over ALL logits.
+// Flags on top of the mode: 4: a group's score is its largest choice value (else the sum of its two largest);
+// 8: the weights are the chosen scores as they are (not divided by their sum).
 template <typename T> struct RouteVec;
 template <> struct RouteVec<float> { static constexpr int N = 4; };
 template <> struct RouteVec<bf16_t> { static constexpr int N = 8; };
@@ -40,8 +42,10 @@ template <typename TX, typename TW, int NT>
 __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x, long x_stride, const TW* __restrict__ wr,
                                                        const float* __restrict__ br, const TW* __restrict__ wg,
                                                        int* __restrict__ idx, float* __restrict__ wt, float* __restrict__ gate,
-                                                       int K, int E, int top, int vec, int mode,
+                                                       int K, int E, int top, int vec, int mode_flags,
                                                        const float* __restrict__ corr, int groups, int keep) {
+    const int mode = mode_flags & 3;
+    const bool group_max = mode_flags & 4, plain_weights = mode_flags & 8;
     extern __shared__ __align__(16) float sm[];        // [K] the row, [E] the logits, [E] the scores, [groups] the groups' scores
     float* xs = sm;
     float* lg = sm + ((K + 3) & ~3);
@@ -69,11 +73,19 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
     }
     __syncthreads();
     if (w != 0) return;
-    if (mode == 1) {
-        // scores s = sigmoid(logit); the choice goes by s + corr among the experts of the `keep` groups (of E / groups
+    if (mode != 0) {
+        float smx = -INFINITY, ssum = 1.f;
+        if (mode == 2) {                               // softmax over all logits: the maximum and the sum, by the wave
+            for (int e = lane; e < E; e += 64) smx = fmaxf(smx, lg[e]);
+            smx = wave_max(smx);
+            float part = 0.f;
+            for (int e = lane; e < E; e += 64) part += expf(lg[e] - smx);
+            ssum = wave_sum(part);
+        }
+        // scores s = sigmoid(logit) (mode 2: the softmax); the choice goes by s + corr among the experts of the `keep` groups (of E / groups
         // neighbours each) whose two largest choice values have the largest sum; the weights are the chosen s, normalised
         for (int e = lane; e < E; e += 64) {
-            const float s = 1.0f / (1.0f + expf(-lg[e]));
+            const float s = mode == 2 ? expf(lg[e] - smx) / ssum : 1.0f / (1.0f + expf(-lg[e]));
             sc[e] = s;
             lg[e] = s + (corr ? corr[e] : 0.f);
         }
@@ -88,7 +100,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
                     const float v = lg[e];
                     if (v > a) { b = a; a = v; } else if (v > b) b = v;
                 }
-                gs[g] = per > 1 ? a + b : a;
+                gs[g] = (per > 1 && !group_max) ? a + b : a;
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -126,7 +138,7 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
             if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
         }
         if (r == 0) mx = best;
-        const float ex = mode == 1 ? sc[bi] : expf(best - mx);
+        const float ex = mode != 0 ? sc[bi] : expf(best - mx);
         sum += ex;
         if (lane == r) { mine = bi; chosen = ex; }
         if (lane == 0) lg[bi] = -INFINITY;
@@ -135,17 +147,17 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x,
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-    if (mode == 1) sum += 1e-20f;
-    if (lane < top) { idx[(size_t)t * top + lane] = mine; wt[(size_t)t * top + lane] = chosen / sum; }
+    if (mode != 0) sum += 1e-20f;
+    if (lane < top) { idx[(size_t)t * top + lane] = mine; wt[(size_t)t * top + lane] = plain_weights ? chosen : chosen / sum; }
 }
 
 extern "C" int li_moe_route(const void* x, int x_dtype, long x_stride, const void* wr, int w_dtype, const float* br, const void* wg,
                             int* idx, float* wt, float* gate, int T, int K, int E, int top, int mode, const float* corr,
                             int groups, int keep, hipStream_t stream) {
-    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (wg && !gate) || mode < 0 || mode > 1 ||
+    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (wg && !gate) || mode < 0 || mode > 15 || (mode & 3) == 3 ||
         groups <= 0 || keep <= 0 || keep > groups || E % groups || (size_t)(K + 2 * E + groups + 4) * 4 > 60000)
         return LI_ERR_SIZE;
-    if (mode == 1 && (long)top > (long)keep * (E / groups)) return LI_ERR_SIZE;      // more choices than the kept groups hold
+    if ((mode & 3) != 0 && (long)top > (long)keep * (E / groups)) return LI_ERR_SIZE;      // more choices than the kept groups hold
     const size_t lds = (size_t)(((K + 3) & ~3) + 2 * E + groups) * 4;
     // whole 16-byte pieces of every matrix row (the gate row included)
     const int ve = w_dtype == LI_F32 ? 4 : 8;
@@ -220,11 +232,21 @@ extern "C" int li_moe_plan(const int* idx, int T, int top, int E, int* plan, int
 }
 
 // Four consecutive outputs of one row, from column `col` (a multiple of 4) on, with the activation: 0 none, 1 max(., 0)^2,
-// 2 the columns are (gate, up) pairs and the two results silu(gate) * up go to columns col / 2 and col / 2 + 1.
+// 2 the columns are (gate, up) pairs and the two results silu(gate) * up go to columns col / 2 and col / 2 + 1;
+// 3 the same pairs with g = min(gate, limit), u = clamp(up, -limit, limit) and the result g sigmoid(1.702 g) (u + 1).
+__device__ __forceinline__ float moe_gated(float g, float u, int act, float limit) {
+    if (act == 3) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return u * (g / (1.0f + expf(-g)));
+}
+
 template <typename TO>
-__device__ __forceinline__ void moe_store4(TO* __restrict__ row, int col, float v0, float v1, float v2, float v3, int act) {
-    if (act == 2) {
-        const float o0 = v1 * (v0 / (1.0f + expf(-v0))), o1 = v3 * (v2 / (1.0f + expf(-v2)));
+__device__ __forceinline__ void moe_store4(TO* __restrict__ row, int col, float v0, float v1, float v2, float v3, int act, float limit) {
+    if (act >= 2) {
+        const float o0 = moe_gated(v0, v1, act, limit), o1 = moe_gated(v2, v3, act, limit);
         TO* dst = row + (col >> 1);
         if constexpr (sizeof(TO) == 2) *reinterpret_cast<uint32_t*>(dst) = pack2_bf16(o0, o1);
         else *reinterpret_cast<float2*>(dst) = float2{o0, o1};
@@ -253,7 +275,7 @@ __device__ __forceinline__ void moe_store4(TO* __restrict__ row, int col, float 
 template <typename TA, typename TW, typename TO>
 __global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                          const TW* __restrict__ w, const int* __restrict__ plan,
-                                                         TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+                                                         TO* __restrict__ out, long out_stride, int n_out, int K, int act, float limit) {
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
@@ -299,9 +321,9 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ 
             const int j = j0 + 2 * tc + (i & 1) + 32 * (i >> 1);
             if (j >= n_out) continue;
             float v = acc[rr][i];
-            if (act == 2) {                            // (gate, up) pairs: i even holds the gate, i + 1 the up value
+            if (act >= 2) {                            // (gate, up) pairs: i even holds the gate, i + 1 the up value
                 if (i & 1) continue;
-                store_from_float(out + (size_t)(r0 + r) * out_stride + (j >> 1), acc[rr][i + 1] * (v / (1.0f + expf(-v))));
+                store_from_float(out + (size_t)(r0 + r) * out_stride + (j >> 1), moe_gated(v, acc[rr][i + 1], act, limit));
                 continue;
             }
             if (act == 1) { v = fmaxf(v, 0.f); v = v * v; }
@@ -320,7 +342,7 @@ union moe_frag8 { uint4 raw; uint32_t w[4]; moe_bf16x8 v; };
 template <typename TA, typename TO>
 __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                               const bf16_t* __restrict__ w, const int* __restrict__ plan,
-                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act, float limit) {
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
@@ -351,7 +373,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const TA* __restri
     TO* orow = out + (size_t)(r0 + ql) * out_stride;
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg)                     // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
-        moe_store4(orow, j0 + 8 * rg + 4 * h2, acc[4 * rg], acc[4 * rg + 1], acc[4 * rg + 2], acc[4 * rg + 3], act);
+        moe_store4(orow, j0 + 8 * rg + 4 * h2, acc[4 * rg], acc[4 * rg + 1], acc[4 * rg + 2], acc[4 * rg + 3], act, limit);
 }
 
 // The wider form, for K a multiple of 32: a wave takes the tile's 32 rows and 128 outputs (four accumulators that
@@ -374,7 +396,7 @@ __device__ __forceinline__ void moe_load_rows(moe_frag8& f, const TA* p) {
 template <typename TA, typename TO, int KSPLIT>
 __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                               const bf16_t* __restrict__ w, const int* __restrict__ plan,
-                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act,
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act, float limit,
                                                               int max_tiles) {
     int tile = blockIdx.x, cb = blockIdx.y;
     if (KSPLIT == 1) {
@@ -464,7 +486,7 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
         const moe_f32x16 c = KSPLIT > 1 ? acc[0] : (f == 0 ? acc[0] : f == 1 ? acc[1] : f == 2 ? acc[2] : acc[3]);
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg)                 // registers 4 rg .. 4 rg + 3: outputs 32 f + 8 rg + 4 h2 ..
-            moe_store4(orow, j0 + 32 * f + 8 * rg + 4 * h2, c[4 * rg], c[4 * rg + 1], c[4 * rg + 2], c[4 * rg + 3], act);
+            moe_store4(orow, j0 + 32 * f + 8 * rg + 4 * h2, c[4 * rg], c[4 * rg + 1], c[4 * rg + 2], c[4 * rg + 3], act, limit);
     }
 }
 
@@ -478,7 +500,7 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
 template <typename TO>
 __global__ __launch_bounds__(256) void moe_linear_rows_kernel(const bf16_t* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                               const bf16_t* __restrict__ w, const int* __restrict__ plan,
-                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act, float limit) {
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
@@ -533,13 +555,10 @@ __global__ __launch_bounds__(256) void moe_linear_rows_kernel(const bf16_t* __re
             for (int r = 0; r < MR_ROWS; ++r) {
                 if (rc + r >= nr) continue;
                 TO* orow = out + (size_t)(r0 + rc + r) * out_stride;
-                if (act == 2) {                        // (gate, up) pairs: n_out is even and j0 a multiple of 4
+                if (act >= 2) {                        // (gate, up) pairs: n_out is even and j0 a multiple of 4
 #pragma unroll
                     for (int j = 0; j < MR_OUT; j += 2)
-                        if (j0 + j < n_out) {
-                            const float g = acc[j][r];
-                            store_from_float(orow + ((j0 + j) >> 1), acc[j + 1][r] * (g / (1.0f + expf(-g))));
-                        }
+                        if (j0 + j < n_out) store_from_float(orow + ((j0 + j) >> 1), moe_gated(acc[j][r], acc[j + 1][r], act, limit));
                     continue;
                 }
 #pragma unroll
@@ -567,7 +586,7 @@ __global__ __launch_bounds__(256) void moe_linear_rows_kernel(const bf16_t* __re
 template <typename TO, int RF>      // RF: row fragments of 32 a wave (1: tiles of 64 rows, 2: of 128)
 __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                              const bf16_t* __restrict__ w, const int* __restrict__ plan,
-                                                             TO* __restrict__ out, long out_stride, int n_out, int K, int act,
+                                                             TO* __restrict__ out, long out_stride, int n_out, int K, int act, float limit,
                                                              int max_tiles) {
     constexpr int MB_ROWS = 64 * RF;
     __shared__ __align__(16) uint16_t As[MB_ROWS * MB_LD];
@@ -671,7 +690,7 @@ __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __res
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg)             // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
                 moe_store4(orow, j0 + 64 * wc + 32 * cf + 8 * rg + 4 * h2, acc[rf][cf][4 * rg], acc[rf][cf][4 * rg + 1],
-                           acc[rf][cf][4 * rg + 2], acc[rf][cf][4 * rg + 3], act);
+                           acc[rf][cf][4 * rg + 2], acc[rf][cf][4 * rg + 3], act, limit);
         }
     }
 }
@@ -682,17 +701,17 @@ extern "C" int li_moe_linear_big_takes(int a_dtype, int w_dtype, int n_out, int 
 }
 
 extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
-                             const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
+                             const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act, float limit,
                              int tile_rows, int rows, hipStream_t stream) {
-    if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || act < 0 || act > 2 || out_stride < (act == 2 ? n_out / 2 : n_out) ||
-        (act == 2 && (n_out & 1)))
+    if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || act < 0 || act > 3 || out_stride < (act >= 2 ? n_out / 2 : n_out) ||
+        (act >= 2 && (n_out & 1)))
         return LI_ERR_SIZE;
     if (tile_rows == MOE_BIG_TILE || tile_rows == MOE_HUGE_TILE) {
         if (!li_moe_linear_big_takes(a_dtype, w_dtype, n_out, K) || a_stride % 8 || out_stride % 4 ||
             ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16)
             return LI_ERR_SIZE;
         const dim3 line((unsigned)((((long)max_tiles * ((n_out + MB_COLS - 1) / MB_COLS) + 63) / 64) * 64));
-#define ML(TO, RF) moe_linear_lds_kernel<TO, RF><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles)
+#define ML(TO, RF) moe_linear_lds_kernel<TO, RF><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, limit, max_tiles)
         const bool huge = tile_rows == MOE_HUGE_TILE;
         if (out_dtype == LI_BF16) { if (huge) ML(bf16_t, 2); else ML(bf16_t, 1); }
         else if (out_dtype == LI_F32) { if (huge) ML(float, 2); else ML(float, 1); }
@@ -706,9 +725,9 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
         ((uintptr_t)a | (uintptr_t)w) % 16 == 0 && (out_dtype == LI_BF16 || out_dtype == LI_F32)) {
         const dim3 grid(max_tiles, (n_out + 4 * MR_OUT - 1) / (4 * MR_OUT));
         if (out_dtype == LI_BF16)
-            moe_linear_rows_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (bf16_t*)out, out_stride, n_out, K, act);
+            moe_linear_rows_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (bf16_t*)out, out_stride, n_out, K, act, limit);
         else
-            moe_linear_rows_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (float*)out, out_stride, n_out, K, act);
+            moe_linear_rows_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (float*)out, out_stride, n_out, K, act, limit);
         return li_launch_status();
     }
     if (w_dtype == LI_BF16 && K % 16 == 0 && n_out % 32 == 0 && a_stride % 8 == 0 && out_stride % 4 == 0 &&
@@ -719,9 +738,9 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
         const dim3 line((unsigned)((((long)max_tiles * ((n_out + 511) / 512) + 63) / 64) * 64));       // whole rounds of eight tiles over eight XCDs
 #define MM(TA, TO)                                                                                                                 \
     {                                                                                                                              \
-        if (split) moe_linear_wide_kernel<TA, TO, 4><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles); \
-        else if (wide) moe_linear_wide_kernel<TA, TO, 1><<<line, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles); \
-        else moe_linear_mfma_kernel<TA, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act); \
+        if (split) moe_linear_wide_kernel<TA, TO, 4><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, limit, max_tiles); \
+        else if (wide) moe_linear_wide_kernel<TA, TO, 1><<<line, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, limit, max_tiles); \
+        else moe_linear_mfma_kernel<TA, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, limit); \
     }
         if (a_dtype == LI_BF16 && out_dtype == LI_BF16) MM(bf16_t, bf16_t)
         else if (a_dtype == LI_BF16 && out_dtype == LI_F32) MM(bf16_t, float)
@@ -732,7 +751,7 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
         return li_launch_status();
     }
     const dim3 grid(max_tiles, (n_out + 63) / 64);
-#define ML(TA, TW, TO) moe_linear_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const TW*)w, plan, (TO*)out, out_stride, n_out, K, act)
+#define ML(TA, TW, TO) moe_linear_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const TW*)w, plan, (TO*)out, out_stride, n_out, K, act, limit)
     if (a_dtype == LI_F32 && w_dtype == LI_F32 && out_dtype == LI_F32) ML(float, float, float);
     else if (a_dtype == LI_BF16 && w_dtype == LI_BF16 && out_dtype == LI_BF16) ML(bf16_t, bf16_t, bf16_t);
     else if (a_dtype == LI_BF16 && w_dtype == LI_BF16 && out_dtype == LI_F32) ML(bf16_t, bf16_t, float);
@@ -744,17 +763,22 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
 }
 
 // ----------------------------------------------------------------------------------------------- the sum
-// x[t, :] += sum_c wt[t, c] * yrow[pair_row[t * top + c], :] (in the order of c) + gate[t] * shared[t, :].
+// x[t, :] += sum_c wt[t, c] * yrow[pair_row[t * top + c], :] (in the order of c) + gate[t] * shared[t, :].  A choice
+// idx[t, c] >= experts (where `ident` is given) is an IDENTITY expert: its output is the token's input row ident[t, :].
+template <typename TI>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long x_stride, const float* __restrict__ yrows,
                                                           long y_stride, const int* __restrict__ pair_row, const float* __restrict__ wt,
                                                           const float* __restrict__ gate, const float* __restrict__ shared_out,
-                                                          long s_stride, int H, int top) {
+                                                          long s_stride, int H, int top, const int* __restrict__ idx, int experts,
+                                                          const TI* __restrict__ ident, long i_stride) {
     const int t = blockIdx.x;
     for (int j = blockIdx.y * 256 + threadIdx.x; j < H; j += gridDim.y * 256) {
         float s = 0.f;
         for (int c = 0; c < top; ++c) {
             const int row = pair_row[(size_t)t * top + c];
             if (row >= 0) s = fmaf(wt[(size_t)t * top + c], yrows[(size_t)row * y_stride + j], s);
+            else if (ident && idx[(size_t)t * top + c] >= experts)
+                s = fmaf(wt[(size_t)t * top + c], load_as_float(ident + (size_t)t * i_stride + j), s);
         }
         if (shared_out) s = fmaf(gate ? gate[t] : 1.f, shared_out[(size_t)t * s_stride + j], s);
         x[(size_t)t * x_stride + j] += s;
@@ -762,10 +786,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
 }
 
 extern "C" int li_moe_combine(float* x, long x_stride, const float* yrows, long y_stride, const int* pair_row, const float* wt,
-                              const float* gate, const float* shared_out, long s_stride, int T, int H, int top, hipStream_t stream) {
-    if (T <= 0 || H <= 0 || top <= 0 || x_stride < H || y_stride < H || (shared_out && s_stride < H)) return LI_ERR_SIZE;
+                              const float* gate, const float* shared_out, long s_stride, int T, int H, int top,
+                              const int* idx, int experts, const void* ident, int ident_dtype, long i_stride, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || top <= 0 || x_stride < H || y_stride < H || (shared_out && s_stride < H) ||
+        (ident && (!idx || i_stride < H || experts < 0)))
+        return LI_ERR_SIZE;
     int ys = (H + 255) / 256;
     if (ys > 64) ys = 64;
-    moe_combine_kernel<<<dim3(T, ys), 256, 0, stream>>>(x, x_stride, yrows, y_stride, pair_row, wt, gate, shared_out, s_stride, H, top);
+    if (ident && ident_dtype == LI_BF16)
+        moe_combine_kernel<bf16_t><<<dim3(T, ys), 256, 0, stream>>>(x, x_stride, yrows, y_stride, pair_row, wt, gate, shared_out, s_stride, H, top,
+                                                                    idx, experts, (const bf16_t*)ident, i_stride);
+    else if (!ident || ident_dtype == LI_F32)
+        moe_combine_kernel<float><<<dim3(T, ys), 256, 0, stream>>>(x, x_stride, yrows, y_stride, pair_row, wt, gate, shared_out, s_stride, H, top,
+                                                                   idx, experts, (const float*)ident, i_stride);
+    else return LI_ERR_DTYPE;
     return li_launch_status();
 }

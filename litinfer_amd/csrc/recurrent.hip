@@ -1,7 +1,8 @@
 // Kernels of recurrent mixers whose state has a fixed size per request: a short causal convolution
 // per channel with its tail of past inputs, the selective state-space recurrence
 //   S_t = a_t S_{t-1} + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t,  a_t = exp(-exp(A_log) dt_t),
-// and the gated RMS norm in groups of columns behind it.  Everything here is float32: inputs, decays,
+// (with `fixed_a`: a_t = fixed_a[head] and dt_t = fixed_dt for every token, a retention with a decay a head),
+// the gated delta rule, and the gated RMS norm in groups of columns behind them.  Everything here is float32: inputs, decays,
 // step sizes, the state and the sums; only the normed output is rounded to the activations' type.
 #include "common.h"
 
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_kernel(
     const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dw,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
     const int* __restrict__ chunk_seg, const int* __restrict__ chunk_idx, float* __restrict__ carry, float* __restrict__ decay,
-    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q) {
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q, const float* __restrict__ fixed_a, float fixed_dt) {
     constexpr int NP = NR * NS, PW = 64 / NS;
     extern __shared__ __align__(16) float lds[];
     float* sB = lds;                                   // [SSM_TB][NP]
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_kernel(
         for (int r = 0; r < NR; ++r) S[r] = 0.f;
     }
     float prod = 1.f;
-    const float Dh = (MODE == 0 && active) ? Dw[head] : 0.f;
+    const float Dh = (MODE == 0 && active && Dw) ? Dw[head] : 0.f;
     for (int b0 = 0; b0 < ntok; b0 += SSM_TB) {
         __syncthreads();
         for (int i = threadIdx.x; i < SSM_TB * NP; i += 64 * SSM_WAVES) {
@@ -182,9 +183,10 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_kernel(
             }
             if (lane < SSM_TB) {
                 const bool ok = b0 + lane < ntok;
-                const float d = ok ? softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]) : 0.f;
+                // (a retention: the same decay and the same step for every token)
+                const float d = !ok ? 0.f : fixed_a ? fixed_dt : softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]);
                 sDt[w * SSM_TB + lane] = d;
-                sA[w * SSM_TB + lane] = expf(-expf(A_log[head]) * d);
+                sA[w * SSM_TB + lane] = fixed_a ? fixed_a[head] : expf(-expf(A_log[head]) * d);
             }
         }
         __syncthreads();
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_quad_kernel(
     const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dw,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
     const int* __restrict__ chunk_seg, const int* __restrict__ chunk_idx, float* __restrict__ carry, float* __restrict__ decay,
-    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q) {
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q, const float* __restrict__ fixed_a, float fixed_dt) {
     constexpr int NP = NR * NS, PW = 256 / NS;
     extern __shared__ __align__(16) float lds[];
     float* sB = lds;                                   // [SSM_TB][NP]
@@ -291,7 +293,7 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_quad_kernel(
         for (int r = 0; r < NR; ++r) S[r] = float4{0.f, 0.f, 0.f, 0.f};
     }
     float prod = 1.f;
-    const float Dh = (MODE == 0 && active) ? Dw[head] : 0.f;
+    const float Dh = (MODE == 0 && active && Dw) ? Dw[head] : 0.f;
     for (int b0 = 0; b0 < ntok; b0 += SSM_TB) {
         __syncthreads();
         for (int i = threadIdx.x; i < SSM_TB * NP; i += 64 * SSM_WAVES) {
@@ -309,9 +311,10 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_quad_kernel(
             }
             if (lane < SSM_TB) {
                 const bool ok = b0 + lane < ntok;
-                const float d = ok ? softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]) : 0.f;
+                // (a retention: the same decay and the same step for every token)
+                const float d = !ok ? 0.f : fixed_a ? fixed_dt : softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]);
                 sDt[w * SSM_TB + lane] = d;
-                sA[w * SSM_TB + lane] = expf(-expf(A_log[head]) * d);
+                sA[w * SSM_TB + lane] = fixed_a ? fixed_a[head] : expf(-expf(A_log[head]) * d);
             }
         }
         __syncthreads();
@@ -424,7 +427,7 @@ template <int NR, int NS, bool QUAD>
 static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride, const float* dt_bias,
                       const float* A_log, const float* Dw, float* state, const int* slots, const int* q_start, const int* q_len,
                       int* chunk_tab, float* carry, float* decay, float* y, long y_stride, int heads, int vdim, int N, int G,
-                      int Q, int segs, int max_chunks, bool chunked, hipStream_t stream) {
+                      int Q, int segs, int max_chunks, bool chunked, const float* fixed_a, float fixed_dt, hipStream_t stream) {
     constexpr int NP = NR * NS, PW = (QUAD ? 256 : 64) / NS;
     const size_t lds = (size_t)(2 * SSM_TB * NP + SSM_WAVES * SSM_TB * PW + 2 * SSM_WAVES * SSM_TB) * sizeof(float);
 #define SSM_KERNEL(MODE_) (QUAD ? ssm_scan_quad_kernel<(QUAD ? NR : 4), (QUAD ? NS : 2), MODE_> : ssm_scan_kernel<(QUAD ? 16 : NR), (QUAD ? 1 : NS), MODE_>)
@@ -432,7 +435,7 @@ static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, lo
     if (!chunked) {
         const dim3 grid(segs, G * ublocks);
         SSM_KERNEL(0)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
-            state, slots, q_start, q_len, nullptr, nullptr, nullptr, nullptr, y, y_stride, heads, vdim, N, G, Q);
+            state, slots, q_start, q_len, nullptr, nullptr, nullptr, nullptr, y, y_stride, heads, vdim, N, G, Q, fixed_a, fixed_dt);
         return li_launch_status();
     }
     int* chunk_seg = chunk_tab;
@@ -441,13 +444,13 @@ static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, lo
     ssm_chunk_index_kernel<<<1, 256, 0, stream>>>(q_len, segs, Q, max_chunks, chunk_seg, chunk_idx, chunk_first);
     const dim3 grid(max_chunks, G * ublocks);
     SSM_KERNEL(1)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
-        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
+        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q, fixed_a, fixed_dt);
     const int NV = N * vdim;
     int zs = (NV + 255) / 256;
     if (zs > 16) zs = 16;
     ssm_carry_kernel<<<dim3(segs, heads, zs), 256, 0, stream>>>(carry, decay, state, slots, q_len, chunk_first, heads, NV, Q);
     SSM_KERNEL(0)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
-        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
+        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q, fixed_a, fixed_dt);
     return li_launch_status();
 #undef SSM_KERNEL
 }
@@ -499,9 +502,9 @@ extern "C" long li_ssm_scan_work_bytes(int T, int segs, int heads, int vdim, int
 extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride, const float* dt_bias,
                            const float* A_log, const float* Dw, float* state, const int* slots, const int* q_start,
                            const int* q_len, float* y, long y_stride, int heads, int vdim, int N, int G, int Q, int T,
-                           int segs, int max_q_len, void* work, long work_bytes, hipStream_t stream) {
+                           int segs, int max_q_len, void* work, long work_bytes, const float* fixed_a, float fixed_dt, hipStream_t stream) {
     if (T <= 0 || segs <= 0 || heads <= 0 || G <= 0 || heads % G || vdim <= 0 || N <= 0 || Q <= 0 || max_q_len <= 0 ||
-        xbc_stride < (long)heads * vdim + 2L * G * N || dt_stride < heads || y_stride < (long)heads * vdim)
+        xbc_stride < (long)heads * vdim + 2L * G * N || (!fixed_a && (dt_stride < heads || !dt_raw || !dt_bias || !A_log)) || y_stride < (long)heads * vdim)
         return LI_ERR_SIZE;
     int ns = 0, nr = 0;
     if (!li_ssm_scan_layout(N, vdim, &ns, &nr)) return LI_ERR_SIZE;
@@ -523,7 +526,7 @@ extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_ra
 #define SSM_QUAD(NR_, NS_)                                                                                                \
     if (qr == NR_ && qs == NS_)                                                                                           \
         return ssm_launch<NR_, NS_, true>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len, \
-                                          chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, stream);
+                                          chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, fixed_a, fixed_dt, stream);
         SSM_QUAD(4, 2) SSM_QUAD(8, 2) SSM_QUAD(16, 2) SSM_QUAD(32, 2)
         SSM_QUAD(4, 4) SSM_QUAD(8, 4) SSM_QUAD(16, 4) SSM_QUAD(32, 4)
         SSM_QUAD(4, 8) SSM_QUAD(8, 8) SSM_QUAD(16, 8) SSM_QUAD(32, 8)
@@ -533,7 +536,7 @@ extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_ra
 #define SSM_GO(NR_, NS_)                                                                                                  \
     if (nr == NR_ && ns == NS_)                                                                                           \
         return ssm_launch<NR_, NS_, false>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len,    \
-                                    chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, stream);
+                                    chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, fixed_a, fixed_dt, stream);
     SSM_GO(16, 1) SSM_GO(32, 1) SSM_GO(64, 1) SSM_GO(128, 1)
     SSM_GO(16, 2) SSM_GO(32, 2) SSM_GO(64, 2) SSM_GO(128, 2)
     SSM_GO(16, 4) SSM_GO(32, 4) SSM_GO(64, 4)
@@ -541,30 +544,241 @@ extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_ra
     return LI_ERR_SIZE;
 }
 
+// ------------------------------------------------------------------------------------ gated delta rule
+// Per head, with a state S of N x vdim values:  S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
+// o_t = S^T q_t (the read-out sees the token's own write).  k_t and q_t are made unit vectors here
+// (x / sqrt(sum x^2 + 1e-6)), q_t times q_scale; beta_t = sigmoid(b_t); g_t = exp(-exp(A_log) softplus(a_t + dt_bias)).
+// Groups of heads share k and q.  A column of the state evolves by itself given the token's k, q, g, beta and its
+// own v, so the layout is the state-space recurrence's: a lane owns CW neighbouring columns x NR state values,
+// the NS slices of a column are neighbouring lanes that add up their shares of S^T k and of S^T q, a wave is
+// 64 CW / NS columns of one head, the four waves of a block belong to ONE group and share k_t and q_t, which lie
+// in LDS DR_TB tokens at a time (normed there: sixteen lanes a token add the squares in a fixed order).
+// Rows of xkq: [v: heads x vdim | k: G x N | q: G x N]; rows of ba: [b: heads | a: heads].
+#define DR_TB 16
+
+template <int NR, int NS, int CW>
+__global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
+    const float* __restrict__ xkq, long x_stride, const float* __restrict__ ba, long ba_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ A_log, float* __restrict__ state,
+    const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, float q_scale) {
+    constexpr int NP = NR * NS, PW = 64 * CW / NS;
+    extern __shared__ __align__(16) float lds[];
+    float* sK = lds;                                   // [DR_TB][NP]
+    float* sQ = sK + DR_TB * NP;                       // [DR_TB][NP]
+    float* sX = sQ + DR_TB * NP;                       // [SSM_WAVES][DR_TB][PW]
+    float* sBeta = sX + SSM_WAVES * DR_TB * PW;        // [SSM_WAVES][DR_TB]
+    float* sG = sBeta + SSM_WAVES * DR_TB;             // [SSM_WAVES][DR_TB]
+    const int seg = blockIdx.x;
+    const int ntok = q_len[seg];
+    if (ntok <= 0) return;
+    const int t0 = q_start[seg];
+    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    const int g = blockIdx.y / ublocks, ub = blockIdx.y % ublocks;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int unit = ub * SSM_WAVES + w;
+    const bool active = unit < U;
+    const int head = g * hpg + (active ? unit / PS : 0), pbase = active ? (unit % PS) * PW : 0;
+    const int pq = lane / NS, s = lane % NS, p = pbase + CW * pq;       // the first of the lane's columns
+    const int inner = heads * vdim;
+    float* st = state + ((size_t)slots[seg] * heads + head) * N * vdim;
+    float S[NR][CW];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int n = s * NR + r;
+        if constexpr (CW == 4) {
+            const float4 v4 = (active && n < N && p < vdim) ? *reinterpret_cast<const float4*>(st + (size_t)n * vdim + p)
+                                                            : float4{0.f, 0.f, 0.f, 0.f};
+            S[r][0] = v4.x; S[r][1] = v4.y; S[r][2] = v4.z; S[r][3] = v4.w;
+        } else {
+#pragma unroll
+            for (int c = 0; c < CW; ++c) S[r][c] = (active && n < N && p + c < vdim) ? st[(size_t)n * vdim + p + c] : 0.f;
+        }
+    }
+    for (int b0 = 0; b0 < ntok; b0 += DR_TB) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < DR_TB * NP; i += 64 * SSM_WAVES) {
+            const int tt = i / NP, n = i % NP;
+            const bool ok = b0 + tt < ntok && n < N;
+            const float* row = xkq + (size_t)(t0 + b0 + tt) * x_stride + inner + (size_t)g * N + n;
+            sK[i] = ok ? row[0] : 0.f;
+            sQ[i] = ok ? row[(size_t)G * N] : 0.f;
+        }
+        if (active) {
+            for (int i = lane; i < DR_TB * PW; i += 64) {
+                const int tt = i / PW, pp = pbase + i % PW;
+                const bool ok = b0 + tt < ntok && pp < vdim;
+                sX[(w * DR_TB + tt) * PW + i % PW] = ok ? xkq[(size_t)(t0 + b0 + tt) * x_stride + (size_t)head * vdim + pp] : 0.f;
+            }
+            if (lane < DR_TB) {
+                const bool ok = b0 + lane < ntok;
+                const float* r2 = ba + (size_t)(t0 + b0 + lane) * ba_stride;
+                sBeta[w * DR_TB + lane] = ok ? 1.0f / (1.0f + expf(-r2[head])) : 0.f;
+                sG[w * DR_TB + lane] = ok ? expf(-expf(A_log[head]) * softplus_f32(r2[heads + head] + dt_bias[head])) : 1.f;
+            }
+        }
+        __syncthreads();
+        {   // unit vectors: token tt = thread / 16, sixteen neighbouring lanes share its N values
+            const int tt = threadIdx.x >> 4, part = threadIdx.x & 15;
+            float sk = 0.f, sq = 0.f;
+            for (int n = part; n < NP; n += 16) {
+                const float kv = sK[tt * NP + n], qv = sQ[tt * NP + n];
+                sk = fmaf(kv, kv, sk);
+                sq = fmaf(qv, qv, sq);
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) {
+                sk += __shfl_xor(sk, o, LI_WAVE);
+                sq += __shfl_xor(sq, o, LI_WAVE);
+            }
+            const float ik = 1.0f / sqrtf(sk + 1e-6f), iq = q_scale / sqrtf(sq + 1e-6f);
+            for (int n = part; n < NP; n += 16) {
+                sK[tt * NP + n] *= ik;
+                sQ[tt * NP + n] *= iq;
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        const int nt = (ntok - b0 < DR_TB) ? ntok - b0 : DR_TB;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float gd = sG[w * DR_TB + tt], beta = sBeta[w * DR_TB + tt];
+            float xv[CW];
+#pragma unroll
+            for (int c = 0; c < CW; ++c) xv[c] = sX[(w * DR_TB + tt) * PW + CW * pq + c];
+            const float4* Kp = reinterpret_cast<const float4*>(sK + tt * NP + s * NR);
+            const float4* Qp = reinterpret_cast<const float4*>(sQ + tt * NP + s * NR);
+            float ks[CW];
+#pragma unroll
+            for (int c = 0; c < CW; ++c) ks[c] = 0.f;
+#pragma unroll
+            for (int r4 = 0; r4 < NR / 4; ++r4) {
+                const float4 kv = Kp[r4];
+                const float kk[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) ks[c] = fmaf(S[4 * r4 + j][c], kk[j], ks[c]);
+            }
+#pragma unroll
+            for (int o = 1; o < NS; o <<= 1)
+#pragma unroll
+                for (int c = 0; c < CW; ++c) ks[c] += __shfl_xor(ks[c], o, LI_WAVE);
+            float u[CW], ov[CW];
+#pragma unroll
+            for (int c = 0; c < CW; ++c) { u[c] = beta * (xv[c] - gd * ks[c]); ov[c] = 0.f; }
+#pragma unroll
+            for (int r4 = 0; r4 < NR / 4; ++r4) {
+                const float4 qv = Qp[r4], kv = Kp[r4];
+                const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, kk[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) {
+                        const float nv = fmaf(gd, S[4 * r4 + j][c], kk[j] * u[c]);
+                        S[4 * r4 + j][c] = nv;
+                        ov[c] = fmaf(nv, qs[j], ov[c]);
+                    }
+            }
+#pragma unroll
+            for (int o = 1; o < NS; o <<= 1)
+#pragma unroll
+                for (int c = 0; c < CW; ++c) ov[c] += __shfl_xor(ov[c], o, LI_WAVE);
+            if (s == 0) {
+                float* yr = y + (size_t)(t0 + b0 + tt) * y_stride + (size_t)head * vdim + p;
+                if constexpr (CW == 4) {
+                    if (p < vdim) *reinterpret_cast<float4*>(yr) = float4{ov[0], ov[1], ov[2], ov[3]};
+                } else {
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) if (p + c < vdim) yr[c] = ov[c];
+                }
+            }
+        }
+    }
+    if (!active) return;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int n = s * NR + r;
+        if (n >= N) continue;
+        if constexpr (CW == 4) {
+            if (p < vdim) *reinterpret_cast<float4*>(st + (size_t)n * vdim + p) = float4{S[r][0], S[r][1], S[r][2], S[r][3]};
+        } else {
+#pragma unroll
+            for (int c = 0; c < CW; ++c) if (p + c < vdim) st[(size_t)n * vdim + p + c] = S[r][c];
+        }
+    }
+}
+
+template <int NR, int NS, int CW>
+static int delta_launch(const float* xkq, long x_stride, const float* ba, long ba_stride, const float* dt_bias, const float* A_log,
+                        float* state, const int* slots, const int* q_start, const int* q_len, float* y, long y_stride,
+                        int heads, int vdim, int N, int G, float q_scale, int segs, hipStream_t stream) {
+    constexpr int NP = NR * NS, PW = 64 * CW / NS;
+    const size_t lds = (size_t)(2 * DR_TB * NP + SSM_WAVES * DR_TB * PW + 2 * SSM_WAVES * DR_TB) * sizeof(float);
+    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    delta_scan_kernel<NR, NS, CW><<<dim3(segs, G * ublocks), 64 * SSM_WAVES, lds, stream>>>(
+        xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, y, y_stride, heads, vdim, N, G, q_scale);
+    return li_launch_status();
+}
+
+// 1 if the recurrence has a layout for a state of N values a column (the state-space recurrence's layouts)
+extern "C" int li_delta_scan_takes(int N, int vdim) { return li_ssm_scan_layout(N, vdim, nullptr, nullptr); }
+
+extern "C" int li_delta_scan(const float* xkq, long x_stride, const float* ba, long ba_stride, const float* dt_bias,
+                             const float* A_log, float* state, const int* slots, const int* q_start, const int* q_len,
+                             float* y, long y_stride, int heads, int vdim, int N, int G, float q_scale, int T, int segs,
+                             hipStream_t stream) {
+    if (T <= 0 || segs <= 0 || heads <= 0 || G <= 0 || heads % G || vdim <= 0 || N <= 0 ||
+        x_stride < (long)heads * vdim + 2L * G * N || ba_stride < 2L * heads || y_stride < (long)heads * vdim)
+        return LI_ERR_SIZE;
+#define DR_ARGS xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, y, y_stride, heads, vdim, N, G, q_scale, segs, stream
+    const bool aligned = ((uintptr_t)state | (uintptr_t)y) % 16 == 0 && y_stride % 4 == 0;
+    int qs = 0, qr = 0;
+    if (aligned && ssm_quad_layout(N, vdim, &qs, &qr)) {
+#define DR_QUAD(NR_, NS_) if (qr == NR_ && qs == NS_) return delta_launch<NR_, NS_, 4>(DR_ARGS);
+        DR_QUAD(4, 2) DR_QUAD(8, 2) DR_QUAD(16, 2) DR_QUAD(32, 2)
+        DR_QUAD(4, 4) DR_QUAD(8, 4) DR_QUAD(16, 4) DR_QUAD(32, 4)
+        DR_QUAD(4, 8) DR_QUAD(8, 8) DR_QUAD(16, 8) DR_QUAD(32, 8)
+        DR_QUAD(4, 16) DR_QUAD(8, 16) DR_QUAD(16, 16)
+#undef DR_QUAD
+    }
+    int ns = 0, nr = 0;
+    if (!li_ssm_scan_layout(N, vdim, &ns, &nr)) return LI_ERR_SIZE;
+#define DR_GO(NR_, NS_) if (nr == NR_ && ns == NS_) return delta_launch<NR_, NS_, 1>(DR_ARGS);
+    DR_GO(16, 1) DR_GO(32, 1) DR_GO(64, 1) DR_GO(128, 1)
+    DR_GO(16, 2) DR_GO(32, 2) DR_GO(64, 2) DR_GO(128, 2)
+    DR_GO(16, 4) DR_GO(32, 4) DR_GO(64, 4)
+#undef DR_GO
+#undef DR_ARGS
+    return LI_ERR_SIZE;
+}
+
 // ------------------------------------------------------------------------------------ gated norm in groups
-// out[t, c] = w[c] * v / sqrt(mean over c's group of v^2 + eps), v = y[t, c] * silu(z[t, c]): the gate comes
-// before the norm; every group of `gs` neighbouring columns has its own root mean square.  A block a (token, group).
+// Every group of `gs` neighbouring columns has its own root mean square.  gate_after 0: out[t, c] = w[c] * v /
+// sqrt(mean of v^2 over c's group + eps) with v = y[t, c] * silu(z[t, c]): the gate comes before the norm.
+// gate_after 1: out[t, c] = w[c] * y / sqrt(mean of y^2 + eps) * silu(z[t, c]): the norm sees y alone.  w null: ones.
+// A block a (token, group).
 template <typename TO, int PER>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, long y_stride,
                                                                const float* __restrict__ z, long z_stride,
                                                                const float* __restrict__ w, float eps, TO* __restrict__ out,
-                                                               long out_stride, int gs) {
+                                                               long out_stride, int gs, int gate_after) {
     __shared__ float red[256 / LI_WAVE];
     const int t = blockIdx.x, c0 = blockIdx.y * gs;
     const float* yr = y + (size_t)t * y_stride + c0;
     const float* zr = z + (size_t)t * z_stride + c0;
-    float v[PER];
+    float v[PER], gt[PER];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const int j = threadIdx.x + i * 256;
-        float g = 0.f;
-        if (j < gs) { const float zz = zr[j]; g = yr[j] * (zz / (1.0f + expf(-zz))); }
+        float g = 0.f, sg = 0.f;
+        if (j < gs) { const float zz = zr[j]; sg = zz / (1.0f + expf(-zz)); g = gate_after ? yr[j] : yr[j] * sg; }
         v[i] = g;
+        gt[i] = gate_after ? sg : 1.f;
         ss += g * g;
     }
     for (int j = threadIdx.x + PER * 256; j < gs; j += 256) {
-        const float zz = zr[j], g = yr[j] * (zz / (1.0f + expf(-zz)));
+        const float zz = zr[j], sg = zz / (1.0f + expf(-zz)), g = gate_after ? yr[j] : yr[j] * sg;
         ss += g * g;
     }
     ss = block_sum<256>(ss, red);
@@ -573,23 +787,24 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __re
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const int j = threadIdx.x + i * 256;
-        if (j < gs) store_from_float(o + j, w[c0 + j] * v[i] * inv);
+        if (j < gs) store_from_float(o + j, (w ? w[c0 + j] : 1.f) * v[i] * inv * gt[i]);
     }
     for (int j = threadIdx.x + PER * 256; j < gs; j += 256) {
-        const float zz = zr[j], g = yr[j] * (zz / (1.0f + expf(-zz)));
-        store_from_float(o + j, w[c0 + j] * g * inv);
+        const float zz = zr[j], sg = zz / (1.0f + expf(-zz)), g = gate_after ? yr[j] : yr[j] * sg;
+        store_from_float(o + j, (w ? w[c0 + j] : 1.f) * g * inv * (gate_after ? sg : 1.f));
     }
 }
 
 extern "C" int li_gated_group_norm(const float* y, long y_stride, const float* z, long z_stride, const float* w, float eps,
-                                   void* out, int out_dtype, long out_stride, int T, int n, int groups, hipStream_t stream) {
+                                   void* out, int out_dtype, long out_stride, int T, int n, int groups, int gate_after,
+                                   hipStream_t stream) {
     if (T <= 0 || n <= 0 || groups <= 0 || n % groups || groups > 65535 || y_stride < n || z_stride < n || out_stride < n)
         return LI_ERR_SIZE;
     const dim3 grid(T, groups);
     if (out_dtype == LI_F32)
-        gated_group_norm_kernel<float, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (float*)out, out_stride, n / groups);
+        gated_group_norm_kernel<float, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (float*)out, out_stride, n / groups, gate_after);
     else if (out_dtype == LI_BF16)
-        gated_group_norm_kernel<bf16_t, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (bf16_t*)out, out_stride, n / groups);
+        gated_group_norm_kernel<bf16_t, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (bf16_t*)out, out_stride, n / groups, gate_after);
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }

@@ -107,6 +107,7 @@ class Model:
             nxt = self.order[i + 1] if i + 1 < len(self.order) else None
             follower = self.layers[nxt.layer] if nxt is not None and nxt.inject is None else None
             stream.next_norm = follower.first_norm() if follower is not None else None
+            stream.next_plain = follower is not None and bool(getattr(follower, "reads_stream_itself", False))
             self.layers[e.layer].forward(stream, ctx, cache.view(i))
             if self.tap is not None:
                 self.tap(i, stream.x)

@@ -37,12 +37,13 @@ _SIGNATURES = {
         "li_kv_store": [P, I, I, I, I, I, P, P, P, I, I, I],
         "li_rope_kv_store": [P, I, I, I, I, I, I, P, P, P, P, P, I, I, I],
         "li_embedding_add": [P, P, P, P, I, P, P, I, I, I],
-        "li_rmsnorm_add": [P, P, F, P, P, F, P, I, I, I],
+        "li_rmsnorm_add": [P, P, F, F, P, F, P, P, F, P, I, I, I, I],
+        "li_gated_act": [P, I, P, I, I, I, I],
         "li_relu_squared": [P, I, P, I, L],
         "li_gelu_gate_rows": [P, P, P, P, P, I, I, I, I, P, I, I, I],
         "li_rope_freq_table": [P, P, I, F, P, P, I],
         "li_rope_pairs_apply": [P, I, I, I, I, I, P, P, I],
-        "li_qk_norm_pairs_store": [P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, I],
+        "li_qk_norm_pairs_store": [P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, I, I],
         "li_latent_norm_pairs_store": [P, L, I, I, I, P, L, I, P, F, P, P, P, P, I, P, I, I, P, L, I, P, P, I, I],
         "li_pair_embedding": [P, P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, L, L],
         "li_layernorm": [P, P, P, F, P, I, I, I],
@@ -55,20 +56,21 @@ _SIGNATURES = {
     },
     "recurrent": {
         "li_causal_conv_silu": [P, L, I, I, P, P, P, P, P, P, P, P, L, I, I, I],
-        "li_ssm_scan": [P, L, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, L],
-        "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I],
+        "li_ssm_scan": [P, L, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, L, P, F],
+        "li_delta_scan": [P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, F, I, I],
+        "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I, I],
     },
     "moe": {
         "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I, I, P, I, I],
         "li_moe_plan": [P, I, I, I, P, I, P, P, I],
-        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, I, I],
-        "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I],
+        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, F, I, I],
+        "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I, P, I, P, I, L],
     },
     "attention_masked": {
-        "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
-        "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
-        "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
-        "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L, P, I, I],
+        "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, P, L, I],
+        "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, P, L, I, P, L],
+        "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, P, L, I, P, L],
+        "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, P, P, L, I, P, L, P, I, I],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, P, L, I, I, P, P],
     },
     "gemm": {
@@ -373,23 +375,40 @@ def embedding_add(out: torch.Tensor, ids: Optional[torch.Tensor] = None, table: 
 
 def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor,
                 next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
-                next_out: Optional[torch.Tensor] = None) -> None:
-    """x += y / sqrt(mean(y^2) + eps) * weight, row by row, in float32; with `next_weight` also
-    next_out = the RMS norm of the new x with those weights and `next_eps`."""
-    _gpu(y, weight, x, next_weight, next_out)
+                next_out: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None,
+                factors=(1.0, 1.0)) -> None:
+    """x += b / sqrt(mean(b^2) + eps) * weight, row by row, in float32, for the branch b = y or, with `y2`,
+    b = factors[0] * y + factors[1] * y2; with `next_weight` also next_out = the RMS norm of the new x with those
+    weights and `next_eps`; with `next_out` alone, next_out = the new x in next_out's type."""
+    _gpu(y, weight, x, next_weight, next_out, y2)
     _chk(y.dim() == 2 and y.shape == x.shape and y.is_contiguous() and x.is_contiguous()
          and y.dtype is torch.float32 and x.dtype is torch.float32, "rmsnorm_add: y and x must be contiguous float32 [T, H]")
+    _chk(y2 is None or (y2.shape == x.shape and y2.is_contiguous() and y2.dtype is torch.float32), "rmsnorm_add: the second branch")
     h = x.shape[1]
     _chk(weight.dtype is torch.float32 and weight.numel() == h and weight.is_contiguous(), "rmsnorm_add: weight")
     if next_weight is not None:
-        _chk(next_out is not None and next_out.shape == x.shape and next_out.is_contiguous() and next_out.dtype in _DT
-             and next_weight.dtype is torch.float32 and next_weight.numel() == h and next_weight.is_contiguous(),
+        _chk(next_out is not None and next_weight.dtype is torch.float32 and next_weight.numel() == h and next_weight.is_contiguous(),
              "rmsnorm_add: the next norm's weight and out")
+    if next_out is not None:
+        _chk(next_out.shape == x.shape and next_out.is_contiguous() and next_out.dtype in _DT, "rmsnorm_add: out of the next reader")
+    nxt = 0 if next_out is None else 1 if next_weight is not None else 2
     if x.shape[0]:
-        _run("elementwise", "li_rmsnorm_add", y.data_ptr(), weight.data_ptr(), float(eps), x.data_ptr(),
-             0 if next_weight is None else next_weight.data_ptr(), float(next_eps),
-             0 if next_weight is None else next_out.data_ptr(), _DT[next_out.dtype] if next_weight is not None else 0,
-             x.shape[0], h)
+        _run("elementwise", "li_rmsnorm_add", y.data_ptr(), 0 if y2 is None else y2.data_ptr(), float(factors[0]), float(factors[1]),
+             weight.data_ptr(), float(eps), x.data_ptr(), 0 if next_weight is None else next_weight.data_ptr(), float(next_eps),
+             0 if next_out is None else next_out.data_ptr(), _DT[next_out.dtype] if next_out is not None else 0, nxt, x.shape[0], h)
+
+
+def gated_act(gate_up: torch.Tensor, out: torch.Tensor, act: str) -> None:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]; act "silu" or "gelu_tanh"; float32 arithmetic; gate_up in
+    float32 or the engine's dtype, out in the engine's."""
+    _gpu(gate_up, out)
+    t, i = out.shape
+    _chk(act in ("silu", "gelu_tanh"), "gated_act: act")
+    _chk(gate_up.shape == (t, 2 * i) and gate_up.is_contiguous() and out.is_contiguous() and gate_up.dtype in _DT and out.dtype in _DT
+         and (gate_up.dtype is torch.float32 or out.dtype is torch.bfloat16), "gated_act: gate_up [T, 2 I], out [T, I]")
+    if t:
+        _run("elementwise", "li_gated_act", gate_up.data_ptr(), _DT[gate_up.dtype], out.data_ptr(), _DT[out.dtype], t, i,
+             1 if act == "gelu_tanh" else 0)
 
 
 def relu_squared(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -453,10 +472,10 @@ def _check_tables(what, t, rotary_dim, cos, sin, slot_map):
 def qk_norm_pairs_store(qkv: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rotary_dim: int,
                         wq: Optional[torch.Tensor], wk: Optional[torch.Tensor], eps: float, cos: torch.Tensor,
                         sin: torch.Tensor, slot_map: Optional[torch.Tensor], k: Optional[torch.Tensor],
-                        v: Optional[torch.Tensor], page_size: int) -> None:
+                        v: Optional[torch.Tensor], page_size: int, half_split: bool = False) -> None:
     """qkv float32 rows [q (nh*dk) | k (nkv*dk) | v (nkv*dv)].  q and k are RMS-normed over their WHOLE
     width (weights wq, wk; None: no norm), their heads' first `rotary_dim` columns rotated in neighbouring
-    pairs; q stays in place, k and v go to their page slots (k None: only q is prepared)."""
+    pairs (`half_split`: column i with column i + rotary_dim / 2); q stays in place, k and v go to their page slots (k None: only q is prepared)."""
     _gpu(qkv, wq, wk, cos, sin, slot_map, k, v)
     t = qkv.shape[0]
     _chk(_rows_ok(qkv) and qkv.dtype is torch.float32 and qkv.shape[1] >= nh * dk + nkv * (dk + dv),
@@ -474,7 +493,8 @@ def qk_norm_pairs_store(qkv: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, 
         _run("elementwise", "li_qk_norm_pairs_store", qkv.data_ptr(), qkv.stride(0), nh, nkv, dk, dv, rotary_dim,
              0 if wq is None else wq.data_ptr(), 0 if wk is None else wk.data_ptr(), float(eps), cos.data_ptr(),
              sin.data_ptr(), 0 if k is None else slot_map.data_ptr(), 0 if k is None else k.data_ptr(),
-             0 if k is None else v.data_ptr(), _DT[k.dtype] if k is not None else 0, page_size, int(k is not None), t)
+             0 if k is None else v.data_ptr(), _DT[k.dtype] if k is not None else 0, page_size, int(k is not None),
+             int(bool(half_split)), t)
 
 
 def latent_norm_pairs_store(qd: Optional[torch.Tensor], nh: int, dn: int, dr: int, rank: int, wc: torch.Tensor, eps: float,
@@ -603,13 +623,17 @@ def _single_blocks(n: int, nh: int, nkv: int, dk: int, dv: int) -> int:
 
 def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, out: torch.Tensor, k: torch.Tensor,
                      v: torch.Tensor, meta, nh: int, nkv: int, dk: int, dv: int, page_size: int, window: int,
-                     keep_first: int, softcap: float, scale: float, ws=None) -> None:
+                     keep_first: int, softcap: float, scale: float, ws=None, sink: Optional[torch.Tensor] = None,
+                     head_gate: Optional[torch.Tensor] = None) -> None:
     """Attention of every token of the step over its request's cached keys: position p sees j <= p with
     p - j < window (0: all) or j < keep_first; scores (q . k) * scale, then softcap * tanh(score / softcap)
     where softcap > 0; softmax and sums in float32.  q: a float32 tensor in which head h of token t starts at
     t * q_token_stride + h * q_head_stride; k [pages, nkv, page, >= dk] and v [pages, nkv, page, >= dv] (the two
-    may be one tensor: then the value is the first dv columns of the key's row); out [T, nh * dv]."""
-    _gpu(q, out, k, v, meta.block_table)
+    may be one tensor: then the value is the first dv columns of the key's row); out [T, nh * dv].
+    `sink` (float32 [nh]): the softmax's denominator also holds exp(sink[head]), a term without key or value.
+    `head_gate` (float32 rows [T, nh], a view of columns is fine): head h's output of token t is multiplied by
+    sigmoid(head_gate[t, h])."""
+    _gpu(q, out, k, v, meta.block_table, sink, head_gate)
     t = out.shape[0]
     _chk(q.dtype is torch.float32 and q.is_contiguous() and q.numel() >= (t - 1) * q_token_stride + (nh - 1) * q_head_stride + dk,
          "masked_attention: q")
@@ -619,6 +643,11 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
          and k.dtype in _DT and (out.dtype is k.dtype or out.dtype is torch.float32), "masked_attention: cache")
     _chk(nh % nkv == 0 and meta.num_tokens == t and meta.block_table.shape == (meta.num_segments, meta.max_blocks),
          "masked_attention: batch")
+    _chk(sink is None or (sink.dtype is torch.float32 and sink.numel() == nh and sink.is_contiguous()), "masked_attention: sink")
+    _chk(head_gate is None or (head_gate.dtype is torch.float32 and _rows_ok(head_gate) and head_gate.shape == (t, nh)),
+         "masked_attention: head_gate")
+    fin = (0 if sink is None else sink.data_ptr(), 0 if head_gate is None else head_gate.data_ptr(),
+           0 if head_gate is None else head_gate.stride(0))
     if not t:
         return
     # keys that one query may see, as far as the host knows without looking at the contexts (a recorded step
@@ -631,7 +660,7 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
              out.data_ptr(), _DT[out.dtype], k.data_ptr(), v.data_ptr(), _DT[k.dtype], k.shape[3], v.shape[3],
              meta.block_table.data_ptr(), meta.max_blocks, 0 if token_list is None else token_list.data_ptr(), n,
              meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
-             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale), waves)
+             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale), *fin, waves)
 
     fast = (k.dtype is torch.bfloat16 and out.dtype is torch.bfloat16 and k.shape[3] % 8 == 0 and v.shape[3] % 8 == 0
             and q_token_stride % 4 == 0 and q_head_stride % 4 == 0 and q.data_ptr() % 16 == 0)
@@ -652,7 +681,7 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
                         meta.block_table.data_ptr(), meta.max_blocks, 0 if token_list is None else token_list.data_ptr(), n,
                         meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
                         nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0),
-                        float(scale), nsplit, parts, parts_n)
+                        float(scale), *fin, nsplit, parts, parts_n)
         if not (fast and masked_single_takes(dk, dv)):
             return general(token_list, n)
         # few blocks against many keys: the keys are cut into splits, each a block of its own, and joined by a second
@@ -670,7 +699,7 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
              out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
              0 if token_list is None else token_list.data_ptr(), n, meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
              meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), nh, nkv, dk, dv, page_size, k.shape[0], int(window),
-             int(keep_first), float(softcap or 0.0), float(scale), nsplit, parts, parts_n)
+             int(keep_first), float(softcap or 0.0), float(scale), *fin, nsplit, parts, parts_n)
 
     if meta.num_single == t and not meta.num_multi:
         return singles(None, t)                                 # a decoding step
@@ -694,7 +723,7 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
              out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
              meta.tiles.data_ptr(), meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale),
-             nsplit, parts, parts_n, 0 if meta.multi_tokens is None else meta.multi_tokens.data_ptr(), n_multi, t)
+             *fin, nsplit, parts, parts_n, 0 if meta.multi_tokens is None else meta.multi_tokens.data_ptr(), n_multi, t)
         if meta.num_single:
             singles(meta.single_tokens, meta.num_single)       # (a list is there: the batch has tokens of both kinds)
         return
@@ -1484,20 +1513,26 @@ def causal_conv_silu(u: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
              out.data_ptr(), out.stride(0), t, ctx.num_segments, int(ctx.max_q_len))
 
 
-def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d: torch.Tensor,
-             state: torch.Tensor, ctx, y: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, ws) -> None:
+def ssm_scan(xbc: torch.Tensor, dt: Optional[torch.Tensor], dt_bias: Optional[torch.Tensor], a_log: Optional[torch.Tensor],
+             d: Optional[torch.Tensor], state: torch.Tensor, ctx, y: torch.Tensor, heads: int, vdim: int, n_state: int,
+             groups: int, ws, fixed_decay: Optional[torch.Tensor] = None, fixed_step: float = 1.0) -> None:
     """The state-space recurrence over each request's tokens of the step, from and into `state`
-    [slots, heads, n_state, vdim] (float32):  S <- exp(-exp(a_log_h) dt) S + dt B x^T,  y = S^T C + d_h x,  with
-    dt = softplus(dt_raw + dt_bias_h).  xbc: float32 rows [x: heads * vdim | B: groups * n_state | C: groups * n_state];
+    [slots, heads, n_state, vdim] (float32):  S <- a S + dt B x^T,  y = S^T C + d_h x,  with a = exp(-exp(a_log_h) dt) and
+    dt = softplus(dt_raw + dt_bias_h), or, with `fixed_decay` (float32 [heads]), a = fixed_decay[h] and dt = fixed_step
+    for every token (dt, dt_bias and a_log are then not read; d None: no x term).
+    xbc: float32 rows [x: heads * vdim | B: groups * n_state | C: groups * n_state];
     dt: float32 rows [heads] (raw); y: float32 rows [heads * vdim].  All float32."""
-    _gpu(xbc, dt, dt_bias, a_log, d, state, y)
+    fixed = fixed_decay is not None
+    _gpu(xbc, dt, dt_bias, a_log, d, state, y, fixed_decay)
     t = y.shape[0]
     inner = heads * vdim
-    _chk(all(x.dtype is torch.float32 for x in (xbc, dt, dt_bias, a_log, d, state, y)), "ssm_scan: everything is float32")
-    _chk(_rows_ok(xbc) and xbc.shape == (t, inner + 2 * groups * n_state) and _rows_ok(dt) and dt.shape == (t, heads)
-         and _rows_ok(y) and y.shape == (t, inner), "ssm_scan: rows")
+    _chk(all(x is None or x.dtype is torch.float32 for x in (xbc, dt, dt_bias, a_log, d, state, y, fixed_decay)), "ssm_scan: everything is float32")
+    _chk(_rows_ok(xbc) and xbc.shape == (t, inner + 2 * groups * n_state) and _rows_ok(y) and y.shape == (t, inner), "ssm_scan: rows")
+    _chk(fixed or (dt is not None and _rows_ok(dt) and dt.shape == (t, heads)
+                   and all(v is not None and v.numel() == heads and v.is_contiguous() for v in (dt_bias, a_log))), "ssm_scan: dt")
+    _chk(not fixed or (fixed_decay.numel() == heads and fixed_decay.is_contiguous()), "ssm_scan: fixed_decay [heads]")
     _chk(state.is_contiguous() and state.shape[1:] == (heads, n_state, vdim) and heads % groups == 0
-         and all(v.numel() == heads and v.is_contiguous() for v in (dt_bias, a_log, d)), "ssm_scan: state [slots, heads, N, vdim]")
+         and (d is None or (d.numel() == heads and d.is_contiguous())), "ssm_scan: state [slots, heads, N, vdim]")
     _chk(ctx.num_tokens == t and int(ctx.host_state_slots.max(initial=0)) < state.shape[0], "ssm_scan: batch")
     _chk(ssm_scan_takes(n_state, vdim), f"ssm_scan: no kernel for a state of {n_state} values a column (at most 256)")
     if not t:
@@ -1508,22 +1543,57 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: 
             t, ctx.num_segments, heads, vdim, n_state, SSM_CHUNK, None)
         buf = ws.buffer("ssm_scan.work", ((int(need) + 3) // 4,), torch.float32)
         work, work_bytes = buf.data_ptr(), buf.numel() * 4
-    _run("recurrent", "li_ssm_scan", xbc.data_ptr(), xbc.stride(0), dt.data_ptr(), dt.stride(0), dt_bias.data_ptr(), a_log.data_ptr(),
-         d.data_ptr(), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(), y.data_ptr(),
-         y.stride(0), heads, vdim, n_state, groups, SSM_CHUNK, t, ctx.num_segments, int(ctx.max_q_len), work, work_bytes)
+
+    def ptr(v):
+        return 0 if v is None else v.data_ptr()
+    _run("recurrent", "li_ssm_scan", xbc.data_ptr(), xbc.stride(0), ptr(dt), 0 if dt is None else dt.stride(0), ptr(dt_bias), ptr(a_log),
+         ptr(d), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(), y.data_ptr(),
+         y.stride(0), heads, vdim, n_state, groups, SSM_CHUNK, t, ctx.num_segments, int(ctx.max_q_len), work, work_bytes,
+         ptr(fixed_decay), float(fixed_step))
 
 
-def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out: torch.Tensor) -> None:
+def delta_scan_takes(n_state: int, vdim: int) -> bool:
+    """Whether the delta-rule kernel has a layout for states of `n_state` values a column."""
+    return bool(_lib_fn("recurrent", "li_delta_scan_takes", [c_int, c_int], c_int)(int(n_state), int(vdim)))
+
+
+def delta_scan(xkq: torch.Tensor, ba: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, ctx,
+               y: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, q_scale: float) -> None:
+    """The gated delta rule over each request's tokens of the step, from and into `state` [slots, heads, n_state, vdim]
+    (float32):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  y = S^T q,  with k and q made unit vectors
+    (x / sqrt(sum x^2 + 1e-6); q times q_scale), beta = sigmoid(b), g = exp(-exp(a_log_h) softplus(a + dt_bias_h)).
+    xkq: float32 rows [v: heads * vdim | k: groups * n_state | q: groups * n_state]; ba: float32 rows [b: heads | a: heads]
+    (raw); y: float32 rows [heads * vdim].  All float32."""
+    _gpu(xkq, ba, dt_bias, a_log, state, y)
+    t = y.shape[0]
+    inner = heads * vdim
+    _chk(all(x.dtype is torch.float32 for x in (xkq, ba, dt_bias, a_log, state, y)), "delta_scan: everything is float32")
+    _chk(_rows_ok(xkq) and xkq.shape == (t, inner + 2 * groups * n_state) and _rows_ok(ba) and ba.shape == (t, 2 * heads)
+         and _rows_ok(y) and y.shape == (t, inner), "delta_scan: rows")
+    _chk(state.is_contiguous() and state.shape[1:] == (heads, n_state, vdim) and heads % groups == 0
+         and all(v.numel() == heads and v.is_contiguous() for v in (dt_bias, a_log)), "delta_scan: state [slots, heads, N, vdim]")
+    _chk(ctx.num_tokens == t and int(ctx.host_state_slots.max(initial=0)) < state.shape[0], "delta_scan: batch")
+    _chk(delta_scan_takes(n_state, vdim), f"delta_scan: no kernel for a state of {n_state} values a column (at most 256)")
+    if t:
+        _run("recurrent", "li_delta_scan", xkq.data_ptr(), xkq.stride(0), ba.data_ptr(), ba.stride(0), dt_bias.data_ptr(),
+             a_log.data_ptr(), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(),
+             y.data_ptr(), y.stride(0), heads, vdim, n_state, groups, float(q_scale), t, ctx.num_segments)
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int, out: torch.Tensor,
+                     gate_after: bool = False) -> None:
     """out = weight * v / sqrt(mean over the group of v^2 + eps), v = y * silu(z), every one of `groups` equal runs of
-    columns by its own mean.  y, z float32 rows; out in either dtype."""
+    columns by its own mean; with `gate_after` the norm sees y alone and its result is multiplied by silu(z).
+    weight None: ones.  y, z float32 rows; out in either dtype."""
     _gpu(y, z, weight, out)
     t, n = out.shape
     _chk(y.dtype is torch.float32 and z.dtype is torch.float32 and _rows_ok(y) and _rows_ok(z) and y.shape == (t, n) and z.shape == (t, n)
-         and _rows_ok(out) and out.dtype in _DT and weight.dtype is torch.float32 and weight.numel() == n and weight.is_contiguous()
+         and _rows_ok(out) and out.dtype in _DT and (weight is None or (weight.dtype is torch.float32 and weight.numel() == n and weight.is_contiguous()))
          and groups > 0 and n % groups == 0, "gated_group_norm: y, z [T, n] float32, weight [n], out [T, n]")
     if t:
-        _run("recurrent", "li_gated_group_norm", y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0), weight.data_ptr(), float(eps),
-             out.data_ptr(), _DT[out.dtype], out.stride(0), t, n, int(groups))
+        _run("recurrent", "li_gated_group_norm", y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0),
+             0 if weight is None else weight.data_ptr(), float(eps), out.data_ptr(), _DT[out.dtype], out.stride(0), t, n, int(groups),
+             int(bool(gate_after)))
 
 
 # --------------------------------------------------------------------------------------- routed feed-forward
@@ -1552,20 +1622,23 @@ def moe_max_tiles(tokens: int, top: int, experts: int, tile_rows: int = MOE_TILE
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], gate_row: Optional[torch.Tensor],
               idx: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor], scores: str = "softmax_chosen",
-              correction: Optional[torch.Tensor] = None, groups: int = 1, keep_groups: int = 1) -> None:
+              correction: Optional[torch.Tensor] = None, groups: int = 1, keep_groups: int = 1,
+              group_score: str = "top2_sum", normalize: bool = True) -> None:
     """idx [T, top] int32: the experts with the largest logits x router^T + bias (float32 sums; the lower index wins a
     tie); wt [T, top] float32: softmax over the chosen logits; gate [T] = sigmoid(x . gate_row) where a row is given.
     With scores = "sigmoid" an expert's score is sigmoid(logit); the choice goes by score + correction[e], and only
     among the experts of the `keep_groups` groups (of experts / groups neighbours each) whose two largest choice
-    values have the largest sum; wt = the chosen scores over their sum (+ 1e-20)."""
+    values have the largest sum (`group_score` = "max": whose largest choice value is largest); wt = the chosen scores
+    over their sum (+ 1e-20), or, with `normalize` False, the chosen scores themselves.  scores = "softmax": the same
+    with an expert's score = the softmax over ALL logits."""
     _gpu(x, router, bias, gate_row, idx, wt, gate, correction)
     t, k = x.shape
     e, top = router.shape[0], idx.shape[1]
-    _chk(scores in ("softmax_chosen", "sigmoid"), "moe_route: scores")
-    mode = 1 if scores == "sigmoid" else 0
-    _chk(correction is None or (mode == 1 and correction.dtype is torch.float32 and correction.numel() == e
+    _chk(scores in ("softmax_chosen", "sigmoid", "softmax") and group_score in ("top2_sum", "max"), "moe_route: scores")
+    mode = {"softmax_chosen": 0, "sigmoid": 1, "softmax": 2}[scores]
+    _chk(correction is None or (mode != 0 and correction.dtype is torch.float32 and correction.numel() == e
                                 and correction.is_contiguous()), "moe_route: correction")
-    _chk(1 <= keep_groups <= groups and e % groups == 0 and (mode == 1 or groups == 1)
+    _chk(1 <= keep_groups <= groups and e % groups == 0 and (mode != 0 or groups == 1)
          and (mode == 0 or top <= keep_groups * (e // groups)), "moe_route: groups")
     _chk(x.dtype in _DT and _rows_ok(x) and router.dtype in _DT and router.is_contiguous() and router.shape == (e, k)
          and (bias is None or (bias.dtype is torch.float32 and bias.numel() == e and bias.is_contiguous())), "moe_route: x, router, bias")
@@ -1577,7 +1650,8 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     if t:
         _run("moe", "li_moe_route", x.data_ptr(), _DT[x.dtype], x.stride(0), router.data_ptr(), _DT[router.dtype],
              0 if bias is None else bias.data_ptr(), 0 if gate_row is None else gate_row.data_ptr(), idx.data_ptr(), wt.data_ptr(),
-             0 if gate is None else gate.data_ptr(), t, k, e, top, mode, 0 if correction is None else correction.data_ptr(),
+             0 if gate is None else gate.data_ptr(), t, k, e, top,
+             mode | (4 if group_score == "max" else 0) | (0 if normalize or mode == 0 else 8), 0 if correction is None else correction.data_ptr(),
              int(groups), int(keep_groups))
 
 
@@ -1600,15 +1674,16 @@ def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: tor
 
 
 def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tensor, plan: torch.Tensor, max_tiles: int,
-               out: torch.Tensor, rows: int, act: int = 0, tile_rows: int = MOE_TILE_ROWS) -> None:
+               out: torch.Tensor, rows: int, act: int = 0, tile_rows: int = MOE_TILE_ROWS, limit: float = 0.0) -> None:
     """out[row] = act(W[expert of the row's tile] a[src(row)]) for the sorted rows of the plan; src(row) = row_token[row]
     where given (rows gathered from tokens), else the row.  w [experts, n_out, K]; act 1: max(., 0)^2; act 2: the
-    matrix rows are (gate, up) pairs, out[row, j] = silu(W[2j] a) * (W[2j + 1] a) and out has n_out / 2 columns."""
+    matrix rows are (gate, up) pairs, out[row, j] = silu(W[2j] a) * (W[2j + 1] a) and out has n_out / 2 columns; act 3:
+    the same pairs with g = min(gate, limit), u = clamp(up, -limit, limit) and out = g sigmoid(1.702 g) (u + 1)."""
     _gpu(a, row_token, w, plan, out)
     e, n_out, k = w.shape
-    _chk(act in (0, 1, 2) and (act != 2 or n_out % 2 == 0), "moe_linear: act")
+    _chk(act in (0, 1, 2, 3) and (act < 2 or n_out % 2 == 0) and (act != 3 or limit > 0), "moe_linear: act")
     _chk(a.dtype in _DT and _rows_ok(a) and a.shape[1] == k and w.dtype in _DT and w.is_contiguous() and out.dtype in _DT and _rows_ok(out)
-         and out.shape == (rows, n_out // 2 if act == 2 else n_out)
+         and out.shape == (rows, n_out // 2 if act >= 2 else n_out)
          and (w.dtype is torch.bfloat16 or (a.dtype is torch.float32 and out.dtype is torch.float32)),
          "moe_linear: a [*, K], w [E, n_out, K], out [rows, n_out]")
     _chk(plan.dtype is torch.int32 and plan.numel() >= 4 + 4 * max_tiles and (row_token is not None or a.shape[0] >= rows)
@@ -1616,13 +1691,16 @@ def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tens
     if rows:
         _run("moe", "li_moe_linear", a.data_ptr(), _DT[a.dtype], a.stride(0), 0 if row_token is None else row_token.data_ptr(),
              w.data_ptr(), _DT[w.dtype], plan.data_ptr(), int(max_tiles), out.data_ptr(), _DT[out.dtype], out.stride(0), n_out, k, int(act),
-             int(tile_rows), int(rows))
+             float(limit), int(tile_rows), int(rows))
 
 
 def moe_combine(x: torch.Tensor, yrows: torch.Tensor, pair_row: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor],
-                shared_out: Optional[torch.Tensor]) -> None:
-    """x[t] += sum_c wt[t, c] * yrows[pair_row[t * top + c]] (in the order of c) + gate[t] * shared_out[t]; float32."""
-    _gpu(x, yrows, pair_row, wt, gate, shared_out)
+                shared_out: Optional[torch.Tensor], idx: Optional[torch.Tensor] = None, experts: int = 0,
+                identity_rows: Optional[torch.Tensor] = None) -> None:
+    """x[t] += sum_c wt[t, c] * yrows[pair_row[t * top + c]] (in the order of c) + gate[t] * shared_out[t]; float32.
+    With `identity_rows` [T, H] (the feed-forward's input), a choice idx[t, c] >= experts is an identity expert whose
+    output is identity_rows[t]."""
+    _gpu(x, yrows, pair_row, wt, gate, shared_out, idx, identity_rows)
     t, h = x.shape
     top = wt.shape[1]
     _chk(x.dtype is torch.float32 and _rows_ok(x) and yrows.dtype is torch.float32 and _rows_ok(yrows) and yrows.shape == (t * top, h)
@@ -1630,7 +1708,12 @@ def moe_combine(x: torch.Tensor, yrows: torch.Tensor, pair_row: torch.Tensor, wt
          and wt.shape[0] == t, "moe_combine: x [T, H], yrows [T * top, H], pair_row, wt")
     _chk(shared_out is None or (shared_out.dtype is torch.float32 and _rows_ok(shared_out) and shared_out.shape == (t, h)
                                 and (gate is None or (gate.dtype is torch.float32 and gate.numel() == t))), "moe_combine: shared")
+    _chk(identity_rows is None or (idx is not None and idx.dtype is torch.int32 and idx.is_contiguous() and idx.shape == (t, top)
+                                   and identity_rows.dtype in _DT and _rows_ok(identity_rows) and identity_rows.shape == (t, h)
+                                   and experts >= 0), "moe_combine: identity experts")
     if t:
         _run("moe", "li_moe_combine", x.data_ptr(), x.stride(0), yrows.data_ptr(), yrows.stride(0), pair_row.data_ptr(), wt.data_ptr(),
              0 if gate is None else gate.data_ptr(), 0 if shared_out is None else shared_out.data_ptr(),
-             0 if shared_out is None else shared_out.stride(0), t, h, top)
+             0 if shared_out is None else shared_out.stride(0), t, h, top,
+             0 if identity_rows is None else idx.data_ptr(), int(experts), 0 if identity_rows is None else identity_rows.data_ptr(),
+             _DT[identity_rows.dtype] if identity_rows is not None else 0, 0 if identity_rows is None else identity_rows.stride(0))

@@ -10,6 +10,9 @@ from .mlp import GeluMLP, ReluSquaredMLP, SwiGLUMLP
 from .moe import RoutedMLP, RoutedReluSquaredMLP
 from .mamba2 import Mamba2Mixer
 from .diff_attention import DiffAttention
+from .delta import GatedDeltaMixer
+from .retention import RetentionMixer
+from .mixer_pair import MixerPair
 from .block import ParallelBlock, PreNormBlock, SandwichBlock
 from .token_side import TokenSideInput
 from .inject import LoopEntry, LoopMix
@@ -19,4 +22,5 @@ __all__ = ["BatchNeeds", "Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed",
            "Part", "Runtime", "StateNeed", "needs_of",
            "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
            "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding", "RopePairs", "BranchStream",
-           "MaskedAttention", "LatentAttention", "RoutedReluSquaredMLP", "Mamba2Mixer", "DiffAttention", "ReluSquaredMLP", "SandwichBlock", "TokenSideInput", "LoopEntry", "LoopMix", "LayerNorm", "GeluMLP", "RoutedMLP", "ParallelBlock", "PairHashEmbedding"]
+           "MaskedAttention", "LatentAttention", "RoutedReluSquaredMLP", "Mamba2Mixer", "DiffAttention", "ReluSquaredMLP", "SandwichBlock", "TokenSideInput", "LoopEntry", "LoopMix", "LayerNorm", "GeluMLP", "RoutedMLP", "ParallelBlock", "PairHashEmbedding", "GatedDeltaMixer",
+           "RetentionMixer", "MixerPair"]

@@ -61,16 +61,18 @@ class SandwichBlock(Block):
     """A norm before AND behind each sublayer: x += norm1b(mixer(norm1(x))), then, if the layer has a
     feed-forward, x += norm2b(ffn(norm2(x))), then, if it has one, the layer's token input
     (`parts/token_side.py`).  A sublayer writes into a branch buffer; the kernel that norms and adds it
-    also leaves the norm through which the stream is read next, where that is known."""
+    also leaves the norm through which the stream is read next, where that is known.
+    The norms BEFORE the sublayers may be absent (no `norm1` / `norm2` among the parts): x += norm1b(mixer(x)),
+    x += norm2b(ffn(x)); the sublayers then read the stream itself, rounded to the parts' dtype."""
 
     def __init__(self, spec, rt, parts):
         super().__init__(spec, rt)
-        self.norm1 = build_part("norm", parts["norm1"], rt)
+        self.norm1 = build_part("norm", parts["norm1"], rt) if parts.get("norm1") is not None else None
         self.mixer = build_part("mixer", parts["mixer"], rt)
         self.norm1b = build_part("norm", parts["norm1b"], rt)
         self.ffn = self.norm2 = self.norm2b = self.token_input = None
         if parts.get("feed_forward") is not None:
-            self.norm2 = build_part("norm", parts["norm2"], rt)
+            self.norm2 = build_part("norm", parts["norm2"], rt) if parts.get("norm2") is not None else None
             self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
             self.norm2b = build_part("norm", parts["norm2b"], rt)
         if parts.get("token_input") is not None:
@@ -104,21 +106,33 @@ class SandwichBlock(Block):
     def first_norm(self):
         return self.norm1
 
+    @property
+    def reads_stream_itself(self):
+        """True if the block's first reader takes the residual sum without a norm."""
+        return self.norm1 is None
+
+    def _read(self, stream, norm, ctx):
+        buf = ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype)
+        return stream.normed(norm, buf) if norm is not None else stream.rounded(buf)
+
     def forward(self, stream, ctx, cache):
         from .stream import BranchStream
-        after = stream.next_norm                   # the norm that reads the stream after this block
-        stream.next_norm = None
-        xn = stream.normed(self.norm1, ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype))
+        after, after_plain = stream.next_norm, stream.next_plain      # who reads the stream after this block
+        stream.next_norm, stream.next_plain = None, False
+        xn = self._read(stream, self.norm1, ctx)
         y = ctx.ws.buffer("block.branch", stream.shape, torch.float32)
         branch = BranchStream(y, ctx.ws)
         self.mixer.forward(xn, branch, ctx, cache)
         last = self.ffn is None and self.token_input is None
-        stream.add_normed(self.norm1b, branch.result(), self.norm2 if self.ffn is not None else (after if last else None))
         if self.ffn is not None:
-            xn = stream.normed(self.norm2, ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype))
+            stream.add_normed(self.norm1b, branch, self.norm2, next_plain=self.norm2 is None)
+            xn = self._read(stream, self.norm2, ctx)
             branch = BranchStream(y, ctx.ws)
             self.ffn.forward(xn, branch, ctx)
-            stream.add_normed(self.norm2b, branch.result(), after if self.token_input is None else None)
+            last = self.token_input is None
+            stream.add_normed(self.norm2b, branch, after if last else None, next_plain=last and after_plain)
+        else:
+            stream.add_normed(self.norm1b, branch, after if last else None, next_plain=last and after_plain)
         if self.token_input is not None:
             self.token_input.forward(stream, ctx, after)
 

@@ -7,7 +7,10 @@ product, left in float32); optionally an RMS norm over the WHOLE of q and the wh
 at once, before the split into heads); the position encoding on the first columns of every query and
 key head; score = (q . k) * scale, then cap * tanh(score / cap) where a cap is given; the query at
 position p sees the keys j <= p with p - j < window (0: all) or j < keep_first; softmax; Wo on the
-heads side by side.
+heads side by side.  Options: biases on q, k and v (`bias`; the tensor's name with `bias_suffix` added); a SINK a
+head (`sink`): the softmax's denominator also holds exp(sink_h), a learned number without key or value; a sigmoid
+gate a head (`head_gate`): head h's output is multiplied by sigmoid(Wg xn)_h before Wo; the position part says how
+it pairs columns (`layout`: neighbouring ones, or column i with column i + rotary_dim/2).
 
 `LatentAttention`: keys and values are expanded from one latent vector c per token, c = the RMS
 norm of the first `rank` rows of Wd xn; the other `rot_dim` rows of Wd xn, rotated, are a key part
@@ -48,16 +51,21 @@ class MaskedAttention(Mixer):
         self.scale = float(a["scale"]) if a.get("scale") is not None else self.dk ** -0.5
         self.qk_norm = bool(a.get("qk_norm", False))
         self.eps = float(a.get("eps", 1e-6))
+        self.bias = bool(a.get("bias", False))
+        self.has_sink = bool(a.get("sink", False))
+        self.head_gate = bool(a.get("head_gate", False))
+        self.gate_cols = -(-int(a["num_heads"]) // 4) * 4 if self.head_gate else 0
         if self.nh <= 0 or self.nkv <= 0 or self.nh % self.nkv:
             raise ValueError(f"attention: {self.nh} heads are not a multiple of {self.nkv} kv heads")
         if self.softcap < 0 or self.window < 0 or self.keep_first < 0:
             raise ValueError("attention: the cap, the window and the kept first positions must not be negative")
         self.position = build_part("position", a["position"], rt) if a.get("position") else None
         self.rotary_dim = int(getattr(self.position, "rotary_dim", 0)) if self.position is not None else 0
-        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm",
-                      **(a.get("names") or {})}
+        self.half_split = getattr(self.position, "layout", "pairs") == "half"
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm", "bias_suffix": ".b",
+                      "sink": "sink", "gate": "g", **(a.get("names") or {})}
         self.n_q, self.n_k, self.n_v = self.nh * self.dk, self.nkv * self.dk, self.nkv * self.dv
-        self.qkv = self.out = self.wq = self.wk = None
+        self.qkv = self.out = self.wq = self.wk = self.sink = None
 
     @property
     def graph_safe(self):
@@ -79,20 +87,37 @@ class MaskedAttention(Mixer):
         if self.qk_norm:
             e[p + n["q_norm"]] = ParamSpec((self.n_q,), init="one_plus_normal")
             e[p + n["k_norm"]] = ParamSpec((self.n_k,), init="one_plus_normal")
+        if self.bias:
+            for x, size in (("q", self.n_q), ("k", self.n_k), ("v", self.n_v)):
+                e[p + n[x] + n["bias_suffix"]] = ParamSpec((size,), init="normal")
+        if self.has_sink:
+            e[p + n["sink"]] = ParamSpec((self.nh,), init="normal")
+        if self.head_gate:
+            e[p + n["gate"]] = ParamSpec((self.nh, self.hidden))
         return e
 
     def load_params(self, get):
         p, n = self.prefix, self.names
         ws = [get(p + n[x]) for x in "qkv"]
+        if self.head_gate:                  # the gates' rows ride behind q, k and v in the one packed product
+            g = get(p + n["gate"])         # (with rows of zeros up to a multiple of four, so that a token's row keeps 16-byte pieces)
+            ws.append(torch.cat([g, torch.zeros(self.gate_cols - self.nh, self.hidden, dtype=g.dtype)], dim=0))
         dt = torch.float32 if any(w.dtype is torch.float32 for w in ws) else ws[0].dtype
-        self.qkv = Linear(self.rt, torch.cat([w.to(dt) for w in ws], dim=0))
+        bias = None
+        if self.bias:
+            bias = torch.cat([get(p + n[x] + n["bias_suffix"]).to(torch.float32) for x in "qkv"]
+                             + ([torch.zeros(self.gate_cols)] if self.head_gate else []))
+        self.qkv = Linear(self.rt, torch.cat([w.to(dt) for w in ws], dim=0), bias)
         self.out = Linear(self.rt, get(p + n["o"]))
+        if self.has_sink:
+            self.sink = self.rt.vector(get(p + n["sink"]))
         if self.qk_norm:
             self.wq, self.wk = self.rt.vector(get(p + n["q_norm"])), self.rt.vector(get(p + n["k_norm"]))
 
     def forward(self, xn, residual, ctx, cache):
         t = xn.shape[0]
-        qkv = ctx.ws.buffer("attn.qkv32", (t, self.n_q + self.n_k + self.n_v), torch.float32)
+        n_qkv = self.n_q + self.n_k + self.n_v
+        qkv = ctx.ws.buffer("attn.qkv32", (t, n_qkv + self.gate_cols), torch.float32)
         self.qkv(xn, qkv, ws=ctx.ws)
         if self.position is not None:
             cos, sin = self.position.tables(ctx)
@@ -101,11 +126,13 @@ class MaskedAttention(Mixer):
         # norm over the whole projections, rotation, and the write of keys and values to their pages: one kernel
         ops.qk_norm_pairs_store(qkv, self.nh, self.nkv, self.dk, self.dv, self.rotary_dim, self.wq, self.wk, self.eps,
                                 cos, sin, ctx.slot_map(cache.group) if cache.owned else None,
-                                cache.k if cache.owned else None, cache.v if cache.owned else None, cache.page_size)
+                                cache.k if cache.owned else None, cache.v if cache.owned else None, cache.page_size,
+                                half_split=self.half_split)
         attn = ctx.ws.buffer("attn.out", (t, self.nh * self.dv), self.rt.dtype)
         ops.masked_attention(qkv, qkv.stride(0), self.dk, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
                              self.nh, self.nkv, self.dk, self.dv, cache.page_size, self.window, self.keep_first,
-                             self.softcap, self.scale, ws=ctx.ws)
+                             self.softcap, self.scale, ws=ctx.ws, sink=self.sink,
+                             head_gate=qkv[:, n_qkv:n_qkv + self.nh] if self.head_gate else None)
         residual.add_linear(self.out, attn)
 
 

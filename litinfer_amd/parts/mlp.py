@@ -1,7 +1,9 @@
 """Dense SwiGLU feed-forward: y = (up * gate / (1 + exp(-gate))) Wd^T with
 gate = xn Wg^T, up = xn Wu^T, no biases (src/llaisys/models/qwen2.cpp:744-759,
 src/ops/swiglu/op.cpp:19-22).  Gate and up are one product with the packed
-matrix [Wg; Wu]; the result is added to the residual stream."""
+matrix [Wg; Wu]; the result is added to the residual stream.  With `activation` = "gelu_tanh" the gate passes the
+tanh form of GELU instead: y = (up * gelu_tanh(gate)) Wd^T; the tensors' names behind the prefix are parameters
+(`names`)."""
 from __future__ import annotations
 
 import torch
@@ -19,29 +21,33 @@ class SwiGLUMLP(FeedForward):
         super().__init__(spec, rt)
         self.hidden = int(spec.args["hidden_size"])
         self.inter = int(spec.args["intermediate_size"])
+        self.activation = str(spec.args.get("activation") or "silu")
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"gated feed-forward: activation {self.activation!r} (silu or gelu_tanh)")
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", **(spec.args.get("names") or {})}
         self.gate_up = None
         self.down = None
 
     def expected_params(self):
-        p = self.prefix
-        return {p + "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
-                p + "up_proj.weight": ParamSpec((self.inter, self.hidden)),
-                p + "down_proj.weight": ParamSpec((self.hidden, self.inter))}
+        p, n = self.prefix, self.names
+        return {p + n["gate"]: ParamSpec((self.inter, self.hidden)),
+                p + n["up"]: ParamSpec((self.inter, self.hidden)),
+                p + n["down"]: ParamSpec((self.hidden, self.inter))}
 
     def batch_needs(self):
         return BatchNeeds(row_tile=self.down.row_tile() if self.down is not None else 1)
 
     def load_params(self, get):
-        p = self.prefix
-        g, u = get(p + "gate_proj.weight"), get(p + "up_proj.weight")
+        p, n = self.prefix, self.names
+        g, u = get(p + n["gate"]), get(p + n["up"])
         dt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
         self.gate_up = Linear(self.rt, torch.cat([g.to(dt), u.to(dt)], dim=0))
-        self.down = Linear(self.rt, get(p + "down_proj.weight"))
+        self.down = Linear(self.rt, get(p + n["down"]))
 
     def forward_prenorm(self, norm, residual, xn, ctx):
         # few rows (decoding): the product before the norm may have left its rows scaled by the
         # norm's weights; the gate/up product then applies the rows' factors with its activation
-        sc = residual.scaled_rows(norm)
+        sc = residual.scaled_rows(norm) if self.activation == "silu" else None
         if sc is not None and self.gate_up.takes_swiglu(sc.rows):
             h = ctx.ws.buffer("mlp.h", (sc.rows.shape[0], self.inter), self.rt.dtype)
             self.gate_up(sc.rows, h, ws=ctx.ws, swiglu=True, row_scale=sc.scale)
@@ -51,16 +57,20 @@ class SwiGLUMLP(FeedForward):
     def forward(self, xn, residual, ctx):
         t = xn.shape[0]
         h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)
-        if self.gate_up.takes_swiglu(xn):
+        if self.activation == "silu" and self.gate_up.takes_swiglu(xn):
             self.gate_up(xn, h, ws=ctx.ws, swiglu=True)        # few rows: the activation is the epilogue
         else:
             gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
             self.gate_up(xn, gu, ws=ctx.ws)
-            ops.swiglu(gu, h)
+            if self.activation == "silu":
+                ops.swiglu(gu, h)
+            else:
+                ops.gated_act(gu, h, self.activation)
         residual.add_linear(self.down, h)
 
 
 register_part("feed_forward", "swiglu_mlp", SwiGLUMLP)
+register_part("feed_forward", "gated_mlp", SwiGLUMLP)
 
 
 class ReluSquaredMLP(FeedForward):

@@ -6,8 +6,13 @@ lower index wins a tie) and weighted by the softmax over the chosen logits alone
 expert's score is sigmoid(logit); the choice goes by score + correction (a stored vector, one number an expert,
 that the weights do not see), and, where the experts form `groups` groups of neighbours, only among the experts of
 the `keep_groups` groups whose two largest choice values have the largest sum; the weights are the chosen scores
-divided by their sum.
-An expert (`activation`): "relu2" is Wdown max(Wup xn, 0)^2; "swiglu" is Wdown (silu(Wgate xn) * (Wup xn)).  No
+divided by their sum.  `scores` = "softmax": the same with an expert's score = the softmax over ALL router outputs.
+`group_score` = "max": a group's score is its largest choice value (default: the sum of its two largest);
+`normalize` False: the weights are the chosen scores as they are.  `identity` > 0: the router has that many outputs
+more than there are experts; the last `identity` of them are identity experts, which have no tensors and whose output
+is the feed-forward's input itself (times the weight); groups are formed over all router outputs.
+An expert (`activation`): "relu2" is Wdown max(Wup xn, 0)^2; "swiglu" is Wdown (silu(Wgate xn) * (Wup xn));
+"clamped_swiglu" is Wdown (g sigmoid(1.702 g) (u + 1)) with g = min(Wgate xn, limit), u = clamp(Wup xn, -limit, limit).  No
 biases.  The shared expert (relu2 only) has a width of its own; its output is multiplied by sigmoid(wg . xn), one
 number a token, where a gate row is given.  The output is the weighted sum, added to the stream in float32.
 
@@ -46,25 +51,35 @@ class RoutedMLP(FeedForward):
         self.keep_groups = int(a.get("keep_groups") or self.groups)
         self.has_correction = bool(a.get("correction", False))
         self.has_router_bias = bool(a.get("router_bias", self.scores == "softmax_chosen"))
+        self.identity = int(a.get("identity") or 0)
+        self.n_router = self.experts + self.identity             # the router's outputs
+        self.group_score = str(a.get("group_score") or "top2_sum")
+        self.normalize = bool(a.get("normalize", True))
+        self.limit = float(a.get("limit") or 0.0)
         self.shared_inter = int(a.get("shared_intermediate_size") or 0)
         self.shared_gate = bool(a.get("shared_gate", True)) and self.shared_inter > 0
-        if min(self.hidden, self.experts, self.top, self.inter) <= 0 or self.top > self.experts:
+        if min(self.hidden, self.experts, self.top, self.inter) <= 0 or self.identity < 0 or self.top > self.n_router:
             raise ValueError(f"routed feed-forward: {self.top} of {self.experts} experts of width {self.inter}")
         if self.top > 64:
             raise ValueError("routed feed-forward: the router kernel picks at most 64 experts a token")
-        if self.activation not in ("relu2", "swiglu") or self.scores not in ("softmax_chosen", "sigmoid"):
-            raise ValueError(f"routed feed-forward: activation {self.activation!r}, scores {self.scores!r}")
-        if self.scores != "sigmoid" and (self.groups != 1 or self.has_correction):
-            raise ValueError("routed feed-forward: groups and a correction of the choice belong to sigmoid scores")
-        if not 1 <= self.keep_groups <= self.groups or self.experts % self.groups:
-            raise ValueError(f"routed feed-forward: {self.experts} experts in {self.groups} groups of which {self.keep_groups} are kept")
-        if self.top > self.keep_groups * (self.experts // self.groups):
+        if (self.activation not in ("relu2", "swiglu", "clamped_swiglu") or self.scores not in ("softmax_chosen", "sigmoid", "softmax")
+                or self.group_score not in ("top2_sum", "max")):
+            raise ValueError(f"routed feed-forward: activation {self.activation!r}, scores {self.scores!r}, group score {self.group_score!r}")
+        if self.activation == "clamped_swiglu" and self.limit <= 0:
+            raise ValueError("routed feed-forward: the clamped activation needs a positive limit")
+        if self.scores == "softmax_chosen" and (self.groups != 1 or self.has_correction or self.identity):
+            raise ValueError("routed feed-forward: groups, a correction of the choice and identity experts belong to "
+                             "scores over all router outputs (sigmoid, softmax)")
+        if not 1 <= self.keep_groups <= self.groups or self.n_router % self.groups:
+            raise ValueError(f"routed feed-forward: {self.n_router} router outputs in {self.groups} groups of which {self.keep_groups} are kept")
+        if self.top > self.keep_groups * (self.n_router // self.groups):
             raise ValueError(f"routed feed-forward: {self.top} choices, but the kept groups hold "
-                             f"{self.keep_groups * (self.experts // self.groups)} experts")
+                             f"{self.keep_groups * (self.n_router // self.groups)} experts")
         if self.shared_inter and self.activation != "relu2":
             raise ValueError("routed feed-forward: the shared expert is a squared-ReLU one")
         self.names = {"expert": "e{}.", "up": "up", "gate": "gate", "down": "down", "router": "router", "router_bias": "router.b",
                       "correction": "correction", "shared": "shared.", "shared_gate": "sg", **(a.get("names") or {})}
+        self.gated = self.activation in ("swiglu", "clamped_swiglu")
         self.w_up = self.w_down = self.router = self.router_b = self.correction = None
         self.gate_row = self.shared_up = self.shared_down = None
 
@@ -73,13 +88,13 @@ class RoutedMLP(FeedForward):
 
     def expected_params(self):
         p, n = self.prefix, self.names
-        out = {p + n["router"]: ParamSpec((self.experts, self.hidden))}
+        out = {p + n["router"]: ParamSpec((self.n_router, self.hidden))}
         if self.has_router_bias:
-            out[p + n["router_bias"]] = ParamSpec((self.experts,), init="zeros")
+            out[p + n["router_bias"]] = ParamSpec((self.n_router,), init="zeros")
         if self.has_correction:
-            out[p + n["correction"]] = ParamSpec((self.experts,), init="normal")
+            out[p + n["correction"]] = ParamSpec((self.n_router,), init="normal")
         for e in range(self.experts):
-            if self.activation == "swiglu":
+            if self.gated:
                 out[self._expert(e, "gate")] = ParamSpec((self.inter, self.hidden))
             out[self._expert(e, "up")] = ParamSpec((self.inter, self.hidden))
             out[self._expert(e, "down")] = ParamSpec((self.hidden, self.inter))
@@ -96,7 +111,7 @@ class RoutedMLP(FeedForward):
 
     def load_params(self, get):
         p, n = self.prefix, self.names
-        if self.activation == "swiglu":      # an expert's gate and up rows in turn: one product, the activation its epilogue
+        if self.gated:                       # an expert's gate and up rows in turn: one product, the activation its epilogue
             first = [torch.stack([get(self._expert(e, "gate")), get(self._expert(e, "up"))], dim=1).reshape(2 * self.inter, self.hidden)
                      for e in range(self.experts)]
         else:
@@ -120,7 +135,8 @@ class RoutedMLP(FeedForward):
         wt = ws.buffer("moe.wt", (t, top), torch.float32)
         gate = ws.buffer("moe.gate", (t,), torch.float32) if self.gate_row is not None else None
         ops.moe_route(xn, self.router, self.router_b, self.gate_row, idx, wt, gate, scores=self.scores,
-                      correction=self.correction, groups=self.groups, keep_groups=self.keep_groups)
+                      correction=self.correction, groups=self.groups, keep_groups=self.keep_groups,
+                      group_score=self.group_score, normalize=self.normalize)
         # (a prompt's portion gives every expert hundreds of rows: larger tiles then, for the kernel that stages them in LDS)
         n_first = self.w_up.shape[1]
         rows_a_tile = ops.moe_tile_rows(t, top, self.experts, xn.dtype, self.w_up.dtype,
@@ -131,8 +147,8 @@ class RoutedMLP(FeedForward):
         pair_row = ws.buffer("moe.pair_row", (pairs,), torch.int32)
         ops.moe_plan(idx, self.experts, plan, row_token, pair_row, rows_a_tile)
         h = ws.buffer("moe.h", (pairs, self.inter), self.rt.dtype)
-        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=2 if self.activation == "swiglu" else 1,
-                       tile_rows=rows_a_tile)
+        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act={"relu2": 1, "swiglu": 2, "clamped_swiglu": 3}[self.activation],
+                       tile_rows=rows_a_tile, limit=self.limit)
         yrows = ws.buffer("moe.y", (pairs, self.hidden), torch.float32)
         ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs, tile_rows=rows_a_tile)
         shared = None
@@ -143,7 +159,9 @@ class RoutedMLP(FeedForward):
             ops.relu_squared(u, hs)
             shared = ws.buffer("moe.shared", (t, self.hidden), torch.float32)
             self.shared_down(hs, shared, ws=ws)
-        ops.moe_combine(residual.tensor(), yrows, pair_row, wt, gate, shared)
+        # (a pair whose choice is an identity expert has no row in the plan: the sum takes the token's input for it)
+        ops.moe_combine(residual.tensor(), yrows, pair_row, wt, gate, shared, idx=idx if self.identity else None,
+                        experts=self.experts, identity_rows=xn if self.identity else None)
 
 
 class RoutedReluSquaredMLP(RoutedMLP):

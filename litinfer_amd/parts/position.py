@@ -116,7 +116,8 @@ class RopePairs(Position):
     original, fast, slow) is the YaRN rule: with dim(t) = rotary_dim ln(original / (2 pi t)) /
     (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rotary_dim - 1) and
     ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency is f_i / factor * ramp_i +
-    f_i (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1.  The frequencies are
+    f_i (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1.  A `scaling` with `kind` = "linear"
+    divides every frequency by `factor` and changes nothing else.  The frequencies are
     worked out once on the host (float64, rounded to float32); the angle, cos and sin are float32.
     With layout "half" the same angles rotate column i with column i + rotary_dim/2 instead."""
     graph_safe = True
@@ -172,6 +173,11 @@ def pair_frequencies(rotary_dim: int, theta: float, scaling=None):
     freq = [theta ** (-2.0 * i / rotary_dim) for i in range(half)]
     if not scaling:
         return freq, 1.0
+    if scaling.get("kind") == "linear":
+        factor = float(scaling["factor"])
+        if factor <= 0:
+            raise ValueError(f"rope scaling: factor must be positive, found {factor}")
+        return [f / factor for f in freq], 1.0
     factor, original = float(scaling["factor"]), float(scaling["original"])
     if factor <= 0 or original <= 0:
         raise ValueError(f"rope scaling: factor and original must be positive, found {factor}, {original}")

@@ -22,11 +22,15 @@ import torch
 from .base import ScaledRows
 
 
+_PLAIN = object()         # in place of a norm: "the sum itself, in the parts' dtype"
+
+
 class ResidualStream:
     def __init__(self, x: torch.Tensor, ws):
         self.x = x
         self.ws = ws
         self.next_norm = None                 # the norm through which the stream is read next, if known
+        self.next_plain = False               # the next reader takes the sum itself, without a norm (known like next_norm)
         self._scaled = None                   # (norm, ScaledRows) left by the last add_linear
         self._normed = None                   # (norm, its result) left by the last add_linear
         self.ws_dtype = torch.bfloat16        # the dtype in which normed rows are handed to the parts (the model sets it)
@@ -69,21 +73,42 @@ class ResidualStream:
         norm.forward(self.x, out)
         return out
 
-    def add_normed(self, norm, y: torch.Tensor, next_norm=None) -> None:
+    def rounded(self, out: torch.Tensor) -> torch.Tensor:
+        """The sum itself as a sublayer without a norm of its own reads it: in the parts' dtype (in `out`, or in the
+        tensor that the last addition already left); in a 32-bit engine the stream's own tensor, which a reader must
+        not write to."""
+        if self._normed is not None and self._normed[0] is _PLAIN:
+            return self._normed[1]
+        if out.dtype is self.x.dtype:
+            return self.x
+        from ..kernels import ops
+        ops.cast(self.x, out)
+        return out
+
+    def add_normed(self, norm, y, next_norm=None, next_plain: bool = False) -> None:
         """x += norm(y) for the output y [T, H] (float32) of a sublayer that is normed BEFORE it joins the
-        stream.  `next_norm`: the norm through which the stream is read next, if the caller knows it; the same
-        kernel then leaves that norm of the new sum, and `normed(next_norm, ...)` hands it out."""
+        stream; y may be the sublayer's `BranchStream`, which can hold two outputs and their factors (the norm then
+        sees factor0 * y0 + factor1 * y1).  `next_norm`: the norm through which the stream is read next, if the
+        caller knows it; the same kernel then leaves that norm of the new sum, and `normed(next_norm, ...)` hands it
+        out.  `next_plain`: the next reader takes the sum itself; the kernel leaves it in the parts' dtype for `rounded`."""
         from ..kernels import ops
         scaling = norm.as_scaling()
         if scaling is None:
             raise NotImplementedError("add_normed: the norm behind a sublayer must be an RMS norm with weights")
+        y2, factors = None, (1.0, 1.0)
+        if isinstance(y, BranchStream):
+            y, y2, factors = y.outputs()
         self._scaled = self._normed = None
         nxt = next_norm.as_scaling() if next_norm is not None else None
-        if nxt is None:
-            ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x)
+        if nxt is None and not (next_plain and self.ws_dtype is not self.x.dtype):
+            ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x, y2=y2, factors=factors)
             return
         rows = self.ws.buffer("stream.normed_rows", self.x.shape, self.ws_dtype)
-        ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x, nxt.weight, nxt.eps, rows)
+        if nxt is None:
+            ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x, None, 0.0, rows, y2=y2, factors=factors)
+            self._normed = (_PLAIN, rows)
+            return
+        ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x, nxt.weight, nxt.eps, rows, y2=y2, factors=factors)
         self._normed = (next_norm, rows)
 
 
@@ -95,6 +120,23 @@ class BranchStream(ResidualStream):
     def __init__(self, y: torch.Tensor, ws):
         super().__init__(y, ws)
         self._fresh = True
+        self.factor = 1.0                    # what this output is multiplied by when it joins
+        self.second = None                   # a second output beside this one (a BranchStream with a factor of its own)
+
+    def fork(self, name: str) -> "BranchStream":
+        """A second output beside this one, for a sublayer made of two that are added with factors."""
+        if self.second is not None:
+            raise NotImplementedError("a branch holds at most two outputs")
+        self.second = BranchStream(self.ws.buffer(name, self.x.shape, torch.float32), self.ws)
+        return self.second
+
+    def outputs(self):
+        """(first output, second output or None, (factor of the first, factor of the second))."""
+        if self.second is None:
+            if self.factor != 1.0:
+                return self.result(), self.result(), (self.factor, 0.0)
+            return self.result(), None, (1.0, 1.0)
+        return self.result(), self.second.result(), (self.factor, self.second.factor)
 
     def tensor(self) -> torch.Tensor:
         if self._fresh:
