@@ -60,11 +60,13 @@ class SwiGLUMLP(FeedForward):
         if self.activation == "silu" and self.gate_up.takes_swiglu(xn):
             self.gate_up(xn, h, ws=ctx.ws, swiglu=True)        # few rows: the activation is the epilogue
         else:
-            gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
-            self.gate_up(xn, gu, ws=ctx.ws)
             if self.activation == "silu":
+                gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
+                self.gate_up(xn, gu, ws=ctx.ws)
                 ops.swiglu(gu, h)
-            else:
+            else:                                              # the product is left in float32 and the activation rounds once
+                gu = ctx.ws.buffer("mlp.gate_up32", (t, 2 * self.inter), torch.float32)
+                self.gate_up(xn, gu, ws=ctx.ws)
                 ops.gated_act(gu, h, self.activation)
         residual.add_linear(self.down, h)
 

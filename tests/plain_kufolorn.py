@@ -165,9 +165,10 @@ def expert(h, w, p, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T
 
 
-def route(h, w, p, r):
+def route(h, w, p, r, margins=None):
     """(chosen router outputs [T, top], their weights [T, top]).  Router outputs experts .. experts + identity - 1
-    are identity experts."""
+    are identity experts.  `margins`, a list, receives per token by how much the last chosen output's choice score
+    beats the best one that is not chosen (infinity where every allowed output is chosen)."""
     n = r["experts"] + r.get("identity", 0)
     z = h @ w[p + "router"].T
     e = np.exp(z - z.max(axis=-1, keepdims=True))
@@ -183,13 +184,17 @@ def route(h, w, p, r):
             for gi in kept[t]:
                 mask[t, gi * per:(gi + 1) * per] = 0.0
         choice = choice + mask
-    idx = np.argsort(-choice, axis=-1, kind="stable")[:, :r["top"]]
+    order = np.argsort(-choice, axis=-1, kind="stable")
+    idx = order[:, :r["top"]]
+    if margins is not None:
+        ranked = np.take_along_axis(choice, order, axis=-1)
+        margins.append(ranked[:, r["top"] - 1] - ranked[:, r["top"]] if r["top"] < n else np.full(h.shape[0], np.inf))
     return idx, np.take_along_axis(s, idx, axis=-1)
 
 
-def moe_ff(h, w, p, mlp):
+def moe_ff(h, w, p, mlp, margins=None):
     r = mlp["router"]
-    idx, wt = route(h, w, p, r)
+    idx, wt = route(h, w, p, r, margins)
     out = np.zeros_like(h)
     for t in range(h.shape[0]):
         for e, a in zip(idx[t], wt[t]):
@@ -201,8 +206,9 @@ def moe_ff(h, w, p, mlp):
 
 
 # ------------------------------------------------------------------------------------------- model
-def forward(cfg, w, ids, taps=None):
-    """Logits [T, vocab] of a whole sequence.  `taps`, a list, receives the stream after every layer."""
+def forward(cfg, w, ids, taps=None, margins=None):
+    """Logits [T, vocab] of a whole sequence.  `taps`, a list, receives the stream after every layer; `margins`, a
+    list, an array [T] for every routed layer: how clear each token's choice of experts was (see `route`)."""
     eps = cfg["norm"]["eps"]
     x = w["embed"][np.asarray(ids)]
     positions = np.arange(len(ids))
@@ -217,7 +223,7 @@ def forward(cfg, w, ids, taps=None):
         x = x + offset_norm(y, w[p + "norm1"], eps)
         mlp = L.get("mlp")
         if mlp is not None:
-            y = dense_ff(x, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(x, w, p + "mlp.", mlp)
+            y = dense_ff(x, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(x, w, p + "mlp.", mlp, margins)
             x = x + offset_norm(y, w[p + "norm2"], eps)
         if taps is not None:
             taps.append(x.copy())

@@ -1,0 +1,385 @@
+"""The Kufolorn decoder on the GPU against the plain implementation (tests/plain_kufolorn.py): whole models of four tiny
+configurations and of configurations drawn at random through the engine's step function (whole prompts, tails decoded
+one by one, portions down to two tokens, mixed batches with pages and slots used again), every layer against the plain
+stream, a standout key far away and at page borders, a state that forgets slowly across portions, slots used again, long
+decoding through recorded steps, greedy generation through the entry point, the scheduler, the command line and the
+trace replay; then every mechanism alone at the level of its kernels."""
+import json
+import math
+import os
+import subprocess
+import sys
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import kufolorn_cases as cases
+import plain_kufolorn as plain
+import schedules
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {"float32": 2e-5, "bfloat16": 6e-2}
+LENGTHS = [5, 17, 33, 70, 150, 41, 64, 2, 1]
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def row_errs(got, ref):
+    return np.abs(got.astype(np.float64) - ref).max(axis=-1) / np.abs(ref).max()
+
+
+def check_rows(out, ref, dt, what):
+    """float32: nine rows in ten within the limit and every row within ten times it.  bfloat16: nine rows in ten, and half of them within half the limit (a
+    router's choice between two experts whose choice values differ by less than the rounding may fall the other way, and
+    moves that token's rows; the sublayers read the stream itself, whose rounding every product sees)."""
+    e = np.concatenate([row_errs(out[r], ref[r]) for r in ref])
+    worst, q90, q50 = float(e.max()), float(np.quantile(e, 0.9)), float(np.quantile(e, 0.5))
+    print(f"[observed] {what} {dt}: worst {worst:.3e}, nine in ten below {q90:.3e}, half below {q50:.3e}")
+    assert q90 < TOL[dt], (what, dt, worst, q90)
+    # (a branch whose output nearly cancels is divided by its small root mean square: single rows of float32 reach 1e-4)
+    assert (worst < 10 * TOL[dt]) if dt == "float32" else (q50 < TOL[dt] / 2), (what, dt, worst, q50)
+    assert np.isfinite(e).all()
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, (cfg, page, seed) in cases.CASES.items():
+        w = cases.draw_weights(cfg, seed)
+        for dt in ("float32", "bfloat16"):
+            d = cases.write_model(tmp_path_factory.mktemp(f"k{name}{dt}"), cfg, w, DT[dt])
+            reqs = helpers.random_requests(cfg["vocab"], LENGTHS, seed + 10)
+            wd = cases.stored(w, DT[dt])
+            out[(name, dt)] = (d, reqs, {r: plain.forward(cfg, wd, t) for r, t in reqs.items()})
+    return out
+
+
+def _engine(d, dt, page, max_tokens, **kw):
+    from litinfer_amd.engine import Engine
+    return Engine.from_dir(d, dtype=dt, device=DEV, page_size=page, max_tokens=max_tokens, max_seqs=4,
+                           page_order_seed=5, **kw)
+
+
+def _rows(eng, rid, toks, cuts):
+    from litinfer_amd.engine import StepEntry
+    return np.concatenate([eng.step([StepEntry(rid, toks[a:b], list(range(b - a)))]).float().cpu().numpy()
+                           for a, b in zip(cuts, cuts[1:]) if b > a])
+
+
+# ------------------------------------------------------------------------------------------ whole models
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(cases.CASES))
+@pytest.mark.parametrize("kind", ["whole", "tail", "chunks", "mixed"])
+def test_schedules_match_the_plain_implementation(models, name, dt, kind):
+    cfg, page, _ = cases.CASES[name]
+    d, reqs, ref = models[(name, dt)]
+    steps = getattr(schedules, kind)(reqs)
+    eng = _engine(d, dt, page, schedules.max_live_tokens(reqs, steps, page if kind == "mixed" else 64))
+    out = schedules.run(eng, reqs, steps)
+    eng.cache.check_invariants()
+    assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+    assert eng.cache.free_slots() == 4
+    if kind == "mixed":
+        assert all(g.pool.total_allocations > g.pool.capacity for g in eng.cache.groups), "no page was used again"
+    check_rows(out, ref, dt, f"{name} {kind}")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Sizes, order of layers, routers and constants drawn from a seed: a mixed schedule on few pages, both dtypes."""
+    cfg = cases.random_config(seed)
+    w32 = cases.draw_weights(cfg, 100 + seed)
+    reqs = helpers.random_requests(cfg["vocab"], [3, 40, 18, 75, 1, 29], 200 + seed)
+    page = (4, 8, 16, 32)[seed % 4]
+    for dt in ("float32", "bfloat16"):
+        d = cases.write_model(tmp_path / dt, cfg, w32, DT[dt])
+        w = cases.stored(w32, DT[dt])
+        ref, clear = {}, {}
+        for r, t in reqs.items():
+            margins = []
+            ref[r] = plain.forward(cfg, w, t, margins=margins)
+            close = np.nonzero(np.min(margins, axis=0) < 0.02)[0] if margins else []
+            clear[r] = int(close[0]) if len(close) else len(t)      # the tokens before a router's first close call
+        steps = schedules.mixed(reqs, seed=seed)
+        eng = _engine(d, dt, page, schedules.max_live_tokens(reqs, steps, page))
+        out = schedules.run(eng, reqs, steps)
+        eng.cache.check_invariants()
+        if dt == "bfloat16":
+            # a choice between two experts that is closer than the rounding of the router's input may fall the other
+            # way, and everything behind that token follows it: only the rows before it are compared
+            out = {r: out[r][:clear[r]] for r in reqs if clear[r]}
+            ref = {r: ref[r][:clear[r]] for r in out}
+            if sum(len(v) for v in ref.values()) < 20:
+                continue
+        check_rows(out, ref, dt, f"random configuration {seed}")
+
+
+@pytest.mark.parametrize("name", list(cases.CASES))
+def test_float32_logits_do_not_depend_on_the_schedule(models, name):
+    cfg, page, _ = cases.CASES[name]
+    d, reqs, _ = models[(name, "float32")]
+    outs = {}
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        steps = getattr(schedules, kind)(reqs)
+        outs[kind] = schedules.run(_engine(d, "float32", page, schedules.max_live_tokens(reqs, steps)), reqs, steps)
+    for kind in ("tail", "chunks", "mixed"):
+        for r in reqs:
+            assert schedules.rel_err(outs[kind][r], outs["whole"][r].astype(np.float64)) < 1e-4, (kind, r)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(cases.CASES))
+def test_every_layer_against_the_plain_stream(models, name, dt):
+    from litinfer_amd.engine import StepEntry
+    cfg, page, seed = cases.CASES[name]
+    d, reqs, _ = models[(name, dt)]
+    w = cases.stored(cases.draw_weights(cfg, seed), DT[dt])
+    toks = reqs["r3"]
+    streams, taps = [], []
+    plain.forward(cfg, w, toks, streams)
+    eng = _engine(d, dt, page, 256)
+    eng.model.tap = lambda i, x: taps.append(x.detach().cpu().numpy().copy())
+    eng.step([StepEntry("a", toks, [0])])
+    assert len(taps) == len(streams) == len(cfg["layers"])
+    for i, (got, ref) in enumerate(zip(taps, streams)):
+        e = np.abs(got - ref).max(axis=-1) / np.abs(ref).max()
+        assert (e.max() if dt == "float32" else np.quantile(e, 0.9)) < TOL[dt], (i, e.max())
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_long_decoding_through_recorded_steps(models, dt):
+    from litinfer_amd.engine import StepEntry
+    cfg, page, seed = cases.CASES["A"]
+    d, _, _ = models[("A", dt)]
+    w = cases.stored(cases.draw_weights(cfg, seed), DT[dt])
+    toks = np.random.default_rng(3).integers(0, cfg["vocab"], 170).tolist()
+    ref = plain.forward(cfg, w, toks)
+    eng = _engine(d, dt, page, 256)
+    rows = [eng.step([StepEntry("a", toks[:20], list(range(20)))]).float().cpu().numpy()]
+    rows += [eng.step([StepEntry("a", [toks[i]], [0])]).float().cpu().numpy().copy() for i in range(20, 170)]
+    assert eng.graph_replays > 100
+    check_rows({"a": np.concatenate(rows)}, {"a": ref}, dt, "150 tokens decoded")
+
+
+def test_slots_that_are_used_again_start_from_zero(models):
+    """Requests follow each other on the same slots: the matrices and the convolution's tail of a finished request must
+    not reach the next one; two requests that take turns keep their own states."""
+    from litinfer_amd.engine import StepEntry
+    cfg, page, _ = cases.CASES["B"]
+    d, reqs, ref = models[("B", "float32")]
+    eng = _engine(d, "float32", page, 1024)
+    for rnd in range(3):
+        for r in ("r0", "r1", "r2", "r5", "r7"):
+            toks = reqs[r]
+            out = _rows(eng, r, toks, [0, 1, len(toks)] if len(toks) > 1 else [0, 1])
+            eng.finish(r)
+            assert schedules.rel_err(out, ref[r]) < 2e-5, (rnd, r)
+    a, b = reqs["r1"], reqs["r2"]
+    got = {"a": [], "b": []}
+    for i in range(12):
+        got["a"].append(eng.step([StepEntry("a", [a[i]], [0])]).float().cpu().numpy().copy())
+        got["b"].append(eng.step([StepEntry("b", [b[i]], [0])]).float().cpu().numpy().copy())
+    assert schedules.rel_err(np.concatenate(got["a"]), ref["r1"][:12]) < 2e-5
+    assert schedules.rel_err(np.concatenate(got["b"]), ref["r2"][:12]) < 2e-5
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_states_that_forget_slowly_across_portions(tmp_path, dt):
+    """Delta heads that decay by less than a hundredth a token and a retention head with decay 0.9995: what the first
+    tokens wrote still counts hundreds of tokens later, across portions cut at 1, 63, 64, 65, 128, 129 tokens."""
+    cfg = {"architecture": "Kufolorn", "vocab": 97, "width": 64, "norm": {"eps": 1e-6},
+           "layers": [cases.delta_layer(4, 2, 32, 16, 3, None),
+                      cases.parallel_layer((2, 1, 16, 16, 0.25, cases.rot(16)), (2, 32, 16, (0.9995, 0.99), cases.rot(8)), 0.2, 1.5, cases.dense(96))]}
+    w32 = cases.draw_weights(cfg, 9, long_memory=True)
+    d = cases.write_model(tmp_path / "m", cfg, w32, DT[dt])
+    w = cases.stored(w32, DT[dt])
+    toks = np.random.default_rng(6).integers(0, 97, 330).tolist()
+    ref = plain.forward(cfg, w, toks)
+    other = list(toks)
+    other[:4] = [(t + 1) % 97 for t in toks[:4]]
+    moved = np.abs(plain.forward(cfg, w, other)[-1] - ref[-1]).max() / np.abs(ref[-1]).max()
+    assert moved > 1000 * TOL["float32"], moved         # the first tokens still count at the end
+    for cuts in ([0, 330], [0, 1, 64, 127, 192, 257, 330], [0, 128, 257, 258, 330], [0, 65, 66, 68, 330]):
+        out = _rows(_engine(d, dt, 16, 512), "a", toks, cuts)
+        check_rows({"a": out}, {"a": ref}, dt, f"slow decay, cuts {cuts}")
+
+
+def test_greedy_generation_through_the_entry_point(models):
+    from litinfer_amd import models as entry
+    cfg, page, seed = cases.CASES["A"]
+    d, reqs, _ = models[("A", "float32")]
+    w = cases.stored(cases.draw_weights(cfg, seed), torch.float32)
+    lm = entry.load(d, dtype="float32", device=DEV, page_size=page, max_tokens=512, max_seqs=4)
+    prompt = reqs["r1"]
+    new = list(lm.generate(prompt, max_new_tokens=12, top_k=1, top_p=1.0, temperature=1.0))
+    assert len(new) == 12
+    seq = list(prompt)
+    for t in new:
+        logits = plain.forward(cfg, w, seq)[-1]
+        top = np.argsort(logits)[::-1]
+        assert t == top[0] or logits[top[0]] - logits[t] < 1e-4 * np.abs(logits).max(), (len(seq), t, top[:3])
+        seq.append(int(t))
+
+
+def test_several_requests_through_the_scheduler(models):
+    """Continuous batching of five prompts on four state slots (tokens are fed back on the device, the scheduler
+    looks ahead): each request's greedy tokens are those of the request alone."""
+    from litinfer_amd import models as entry
+    cfg, page, seed = cases.CASES["C"]
+    d, reqs, _ = models[("C", "float32")]
+    lm = entry.load(d, dtype="float32", device=DEV, page_size=page, max_tokens=1024, max_seqs=4)
+    prompts = [reqs[r] for r in ("r0", "r1", "r2", "r5", "r7")]
+    alone = [list(lm.generate(p, max_new_tokens=8)) for p in prompts]
+    lm.engine_start()
+    ids = [lm.engine_add_request(p, 8) for p in prompts]
+    while lm.engine_has_unfinished():
+        lm.engine_step()
+    got = {i: list(lm.engine_get_output(i)) for i in ids}
+    assert [got[i] for i in ids] == alone
+
+
+def test_generate_through_the_command_line(models):
+    cfg, page, seed = cases.CASES["D"]
+    d, reqs, _ = models[("D", "float32")]
+    w = cases.stored(cases.draw_weights(cfg, seed), torch.float32)
+    prompt = reqs["r1"]
+    r = subprocess.run([sys.executable, "-m", "litinfer_amd", "generate", "--model", str(d), "--dtype", "float32", "--prompt-ids",
+                        ",".join(map(str, prompt)), "--max-new-tokens", "6", "--top-k", "1"], cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    seq = list(prompt)
+    for _ in range(6):
+        seq.append(int(np.argmax(plain.forward(cfg, w, seq)[-1])))
+    assert ",".join(map(str, seq[len(prompt):])) in r.stdout.replace(" ", ""), r.stdout[-500:]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_trace_replay_in_a_subprocess(models, tmp_path, dt):
+    cfg, page, _ = cases.CASES["A"]
+    d, reqs, ref = models[("A", dt)]
+    use = {r: reqs[r] for r in ("r0", "r1", "r3", "r5", "r7")}
+    steps = schedules.mixed(use, seed=2)
+    lines = []
+    for n, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": n, "entries": [{"id": r, "tokens": use[r][i:i + k], "want": list(range(k))} for r, i, k in entries],
+                                 "end": end}))
+    out = tmp_path / "out"
+    r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", str(d), "--dtype", dt, "--out", str(out), "--max-tokens",
+                        str(schedules.max_live_tokens(use, steps, 64))], input="\n".join(lines) + "\n", cwd=ROOT, capture_output=True,
+                       text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {n}" for n in range(len(steps))]
+    rows = {r_: [] for r_ in use}
+    for n, (entries, end) in enumerate(steps):
+        a = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"])
+        o = 0
+        for r_, i, k in entries:
+            rows[r_].append(a[o:o + k])
+            o += k
+    check_rows({r_: np.concatenate(v) for r_, v in rows.items()}, {r_: ref[r_] for r_ in use}, dt, "trace replay")
+
+
+# ------------------------------------------------------------------------------------------- a standout key
+def _standout_model(tmp, dt, sink=0.0):
+    """A parallel layer (and a delta layer behind it) whose weights make ONE key win: token A's key scores e^14 with
+    token B's query in every head, through the columns that are not rotated, and A's value is large.  Whether B sees A
+    decides B's logits.  The norm over the whole projections keeps the direction, so the score is set through the norm's
+    known result: unit root mean square."""
+    heads, kvh, dk, dv, scale = 4, 2, 16, 16, 0.5
+    cfg = {"architecture": "Kufolorn", "vocab": 64, "width": 64, "norm": {"eps": 1e-6},
+           "layers": [cases.parallel_layer((heads, kvh, dk, dv, scale, cases.rot(4)), (1, 8, 8, (0.5,), cases.rot(8)), 1.0, 0.05, None),
+                      cases.delta_layer(2, 1, 8, 8, 2, cases.dense(48))]}
+    w = cases.draw_weights(cfg, 5)
+    A, B = 63, 62
+    p = "l0.mix.left."
+    w["embed"][:, :2] = 0.0
+    w["embed"][A] = 0.0
+    w["embed"][B] = 0.0
+    w["embed"][A, 0] = w["embed"][B, 1] = 3.0
+    for n in ("q", "k"):
+        w[p + n] *= 0.02
+        w[p + n + ".b"][:] = 0.0
+        w[p + n + ".norm"][:] = 1.0
+    w[p + "sink"][:] = sink
+    rng = np.random.default_rng(1)
+    # A's key and B's query: the same direction u (over the columns 4.. of every head, which are not rotated); after the
+    # norm over the whole projection each has root mean square 1, so |k|^2 = kvh * dk, |q|^2 = heads * dk, and a head's
+    # score is scale * (dk-4 shared columns) * (root mean square 1 each, about) ~ scale * |u_h|^2
+    for n, hh in (("k", kvh), ("q", heads)):
+        for h in range(hh):
+            w[p + n][h * dk + 4:(h + 1) * dk, 0 if n == "k" else 1] = 1.0
+    w[p + "v"][:, 0] += 6.0 * rng.normal(size=kvh * dv)
+    d = cases.write_model(tmp, cfg, w, DT[dt])
+    return cfg, cases.stored(w, DT[dt]), d, A, B
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds(tmp_path, dt):
+    from litinfer_amd.engine import StepEntry
+    cfg, w, d, A, B = _standout_model(tmp_path / "m", dt)
+    rng = np.random.default_rng(4)
+    toks = rng.integers(0, 60, 420).tolist()
+    toks[3], toks[400] = A, B
+    ref = plain.forward(cfg, w, toks)
+    other = list(toks)
+    other[3] = 5
+    assert np.abs(plain.forward(cfg, w, other)[400] - ref[400]).max() > 0.1 * np.abs(ref[400]).max()
+    for cuts in ([0, 420], [0, 390, 420], [0, 2, 5, 399, 401, 420]):
+        out = _rows(_engine(d, dt, 16, 512), "a", toks, cuts)
+        assert schedules.rel_err(out[395:], ref[395:]) < TOL[dt], cuts
+    eng = _engine(d, dt, 16, 512)
+    eng.step([StepEntry("a", toks[:398], [])])
+    out = np.concatenate([eng.step([StepEntry("a", [toks[i]], [0])]).float().cpu().numpy().copy() for i in range(398, 404)])
+    assert schedules.rel_err(out, ref[398:404]) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("how", ["prompt", "portions", "decoded"])
+def test_a_key_at_page_borders_at_the_query_and_behind_it(tmp_path, dt, how):
+    """The key at the last and the first row of a page and at position 0; the query right behind the key, many pages
+    later, and BEFORE it (the key must not be seen: the rows then equal those of a sequence without it)."""
+    from litinfer_amd.engine import StepEntry
+    cfg, w, d, A, B = _standout_model(tmp_path / "m", dt)
+    rng = np.random.default_rng(3)
+    page, moved = 8, []
+    for pa, pb in ((0, 70), (7, 8), (8, 71), (15, 16), (16, 95), (31, 33), (40, 39)):
+        toks = rng.integers(0, 60, max(pa, pb) + 4).tolist()
+        toks[pa], toks[pb] = A, B
+        ref = plain.forward(cfg, w, toks)
+        without = list(toks)
+        without[pa] = 7
+        moved.append(np.abs(plain.forward(cfg, w, without)[pb] - ref[pb]).max() / np.abs(ref[pb]).max())
+        eng = _engine(d, dt, page, 128)
+        n = len(toks)
+        if how == "prompt":
+            out = _rows(eng, "a", toks, [0, n])
+        elif how == "portions":                                  # a cut between the two, one right at the later one, portions of two
+            lo, hi = min(pa, pb), max(pa, pb)
+            out = _rows(eng, "a", toks, sorted({0, lo + 1, hi, hi + 2, n}))
+        else:
+            head = min(pa, pb) + 1
+            rows = [eng.step([StepEntry("a", toks[:head], list(range(head)))]).float().cpu().numpy()]
+            rows += [eng.step([StepEntry("a", [toks[i]], [0])]).float().cpu().numpy().copy() for i in range(head, n)]
+            out = np.concatenate(rows)
+        assert schedules.rel_err(out, ref) < TOL[dt], (pa, pb)
+    # the test has teeth: the key, where it is seen, moves the query's logits by far more than the tolerance
+    assert min(moved[:-1]) > 0.1, moved
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_a_sink_that_outweighs_every_key(tmp_path, dt):
+    """With a large sink nearly all of the softmax's weight goes to the term without a value: the attention's output
+    shrinks towards zero.  Leaving the sink out, or counting it once a split of the keys, changes the logits by far more
+    than the tolerance."""
+    cfg, w, d, A, B = _standout_model(tmp_path / "m", dt, sink=6.0)
+    toks = np.random.default_rng(8).integers(0, 60, 300).tolist()
+    ref = plain.forward(cfg, w, toks)
+    w0 = dict(w)
+    w0["l0.mix.left.sink"] = w["l0.mix.left.sink"] - 50.0
+    assert np.abs(plain.forward(cfg, w0, toks) - ref).max() > 0.1 * np.abs(ref).max()
+    for cuts in ([0, 300], [0, 290, 291, 292, 300], [0, 33, 35, 300]):
+        out = _rows(_engine(d, dt, 16, 512), "a", toks, cuts)
+        check_rows({"a": out}, {"a": ref}, dt, f"large sink, cuts {cuts}")
