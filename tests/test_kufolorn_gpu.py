@@ -383,3 +383,277 @@ def test_a_sink_that_outweighs_every_key(tmp_path, dt):
     for cuts in ([0, 300], [0, 290, 291, 292, 300], [0, 33, 35, 300]):
         out = _rows(_engine(d, dt, 16, 512), "a", toks, cuts)
         check_rows({"a": out}, {"a": ref}, dt, f"large sink, cuts {cuts}")
+
+
+# ------------------------------------------------------------------------------------------ mechanisms alone
+def _ctx(q_lens, slots):
+    q_len = np.asarray(q_lens, dtype=np.int32)
+    q_start = np.concatenate([[0], np.cumsum(q_len)[:-1]]).astype(np.int32)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(DEV)
+    return SimpleNamespace(num_tokens=int(q_len.sum()), num_segments=len(q_len), host_state_slots=np.asarray(slots, dtype=np.int32),
+                           seg_of_token=dev(np.repeat(np.arange(len(q_len)), q_len)), q_start=dev(q_start), q_len=dev(q_len),
+                           state_slots=dev(slots), max_q_len=int(q_len.max()))
+
+
+def _f32(a):
+    return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV)
+
+
+STEPS = ([(0, 1), (2, 5)], [(2, 1), (0, 2)], [(0, 1)], [(0, 20), (2, 2)], [(2, 15), (0, 16)], [(2, 100), (0, 1)], [(0, 99), (2, 1)])
+
+
+@pytest.mark.parametrize("heads,groups,N,vdim", [(6, 3, 24, 16), (2, 2, 8, 40), (4, 2, 128, 64), (8, 8, 64, 32), (12, 3, 16, 20),
+                                                 (1, 1, 256, 8), (2, 1, 32, 128), (3, 1, 100, 6), (2, 2, 128, 128)])
+def test_delta_rule_across_steps_and_slots(heads, groups, N, vdim):
+    """Two requests on slots 0 and 2 take turns with portions of 1 to 100 tokens; slot 1 is nobody's and stays as it is."""
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(N + vdim)
+    inner, rep = heads * vdim, heads // groups
+    a_log, dt_bias = rng.uniform(-3, 0, heads), rng.normal(0, 0.5, heads)
+    seqs, ref = {}, {}
+    for s in (0, 2):
+        L = 140 if s == 0 else 124
+        v, k, q = rng.normal(size=(L, heads, vdim)), rng.normal(size=(L, groups, N)), rng.normal(size=(L, groups, N))
+        b, a = rng.normal(size=(L, heads)), rng.normal(size=(L, heads))
+        seqs[s] = (np.concatenate([v.reshape(L, -1), k.reshape(L, -1), q.reshape(L, -1)], axis=1), np.concatenate([b, a], axis=1))
+        g = np.exp(-np.exp(a_log) * plain.softplus(a + dt_bias))
+        ref[s] = plain.delta_rule(np.repeat(plain.unit(q) * N ** -0.5, rep, axis=1), np.repeat(plain.unit(k), rep, axis=1), v,
+                                  plain.sigmoid(b), g).reshape(L, inner)
+    state = torch.zeros(3, heads, N, vdim, device=DEV)
+    state[1] = 7.0
+    at = {0: 0, 2: 0}
+    for step in STEPS:
+        x = np.concatenate([seqs[s][0][at[s]:at[s] + n] for s, n in step])
+        ba = np.concatenate([seqs[s][1][at[s]:at[s] + n] for s, n in step])
+        wide = torch.zeros(len(x), ba.shape[1] + 3, device=DEV)                 # (the rows of b and a lie inside a wider buffer)
+        wide[:, 3:] = _f32(ba)
+        y = torch.empty(len(x), inner, device=DEV)
+        ops.delta_scan(_f32(x), wide[:, 3:], _f32(dt_bias), _f32(a_log), state, _ctx([n for _, n in step], [s for s, _ in step]),
+                       y, heads, vdim, N, groups, N ** -0.5)
+        want = np.concatenate([ref[s][at[s]:at[s] + n] for s, n in step])
+        assert np.abs(y.cpu().numpy() - want).max() < 2e-5 * max(1.0, np.abs(want).max()), step
+        for s, n in step:
+            at[s] += n
+    assert torch.all(state[1] == 7.0)
+
+
+@pytest.mark.parametrize("heads,N,vdim", [(3, 12, 20), (2, 64, 32), (4, 128, 64), (1, 20, 8), (2, 16, 16)])
+def test_retention_is_the_recurrence_with_a_fixed_decay(heads, N, vdim):
+    """Portions up to 100 tokens (chunks that run side by side) and single tokens, on two slots."""
+    from litinfer_amd.engine.workspace import Workspace
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(N)
+    decay = rng.uniform(0.8, 0.9995, heads)
+    seqs, ref = {}, {}
+    for s in (0, 2):
+        L = 140 if s == 0 else 124
+        v, k, q = rng.normal(size=(L, heads, vdim)), rng.normal(size=(L, heads, N)), rng.normal(size=(L, heads, N))
+        seqs[s] = np.concatenate([v.reshape(L, -1), k.reshape(L, -1), q.reshape(L, -1)], axis=1)
+        out = np.zeros((L, heads, vdim))
+        for h in range(heads):
+            S = np.zeros((N, vdim))
+            for t in range(L):
+                S = decay[h] * S + np.outer(k[t, h], v[t, h]) * N ** -0.5
+                out[t, h] = S.T @ q[t, h]
+        ref[s] = out.reshape(L, -1)
+    state = torch.zeros(3, heads, N, vdim, device=DEV)
+    ws, at = Workspace(DEV), {0: 0, 2: 0}
+    for step in STEPS:
+        x = np.concatenate([seqs[s][at[s]:at[s] + n] for s, n in step])
+        y = torch.empty(len(x), heads * vdim, device=DEV)
+        ops.ssm_scan(_f32(x), None, None, None, None, state, _ctx([n for _, n in step], [s for s, _ in step]), y, heads, vdim, N,
+                     heads, ws, fixed_decay=_f32(decay), fixed_step=N ** -0.5)
+        want = np.concatenate([ref[s][at[s]:at[s] + n] for s, n in step])
+        assert np.abs(y.cpu().numpy() - want).max() < 2e-5 * max(1.0, np.abs(want).max()), step
+        for s, n in step:
+            at[s] += n
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_small_kernels_of_the_design(dt):
+    """The norm behind a recurrence with its gate BEHIND the norm (with and without weights), the gated tanh GELU, and
+    the kernel that norms a branch of two outputs with factors, adds it and leaves the new sum for the next reader."""
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(0)
+    tol = 1e-5 if dt == "float32" else 1e-2
+    T, heads, vdim = 37, 5, 24
+    y, z, w = rng.normal(size=(T, heads * vdim)), rng.normal(size=(T, heads * vdim)), rng.normal(1, 0.2, heads * vdim)
+    for weights in (w, None):
+        out = torch.empty(T, heads * vdim, dtype=DT[dt], device=DEV)
+        ops.gated_group_norm(_f32(y), _f32(z), None if weights is None else _f32(weights), 1e-3, heads, out, gate_after=True)
+        want = plain.rms(y.reshape(T, heads, vdim), 1e-3).reshape(T, -1) * (1.0 if weights is None else weights) * plain.silu(z)
+        assert np.abs(out.float().cpu().numpy() - want).max() < tol * np.abs(want).max()
+    I = 100
+    gu = rng.normal(0, 2, size=(T, 2 * I))
+    out = torch.empty(T, I, dtype=DT[dt], device=DEV)
+    ops.gated_act(_f32(gu), out, "gelu_tanh")
+    want = plain.gelu_tanh(gu[:, :I]) * gu[:, I:]
+    assert np.abs(out.float().cpu().numpy() - want).max() < tol * np.abs(want).max()
+    H = 72
+    x, y1, y2, w1 = rng.normal(size=(T, H)), rng.normal(size=(T, H)), rng.normal(size=(T, H)), rng.normal(1, 0.2, H)
+    xd, rows = _f32(x), torch.empty(T, H, dtype=DT[dt], device=DEV)
+    ops.rmsnorm_add(_f32(y1), _f32(w1), 1e-4, xd, None, 0.0, rows, y2=_f32(y2), factors=(0.6, -1.5))
+    want = x + plain.rms(0.6 * y1 - 1.5 * y2, 1e-4) * w1
+    assert np.abs(xd.cpu().numpy() - want).max() < 1e-5 * np.abs(want).max()
+    assert np.abs(rows.float().cpu().numpy() - want).max() < tol * np.abs(want).max()
+
+
+@pytest.mark.parametrize("nh,nkv,dk,dv,rot", [(4, 2, 24, 16, 8), (8, 4, 64, 64, 64), (1, 1, 8, 8, 2), (6, 6, 10, 30, 10), (3, 1, 128, 64, 32)])
+def test_norm_over_the_whole_projections_and_half_split_rotation(nh, nkv, dk, dv, rot):
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(dk)
+    T, page = 19, 8
+    qkv = rng.normal(size=(T, nh * dk + nkv * (dk + dv) + 4))              # (the gates' columns ride behind)
+    wq, wk = rng.normal(1, 0.2, nh * dk), rng.normal(1, 0.2, nkv * dk)
+    pos = np.arange(40, 40 + T)
+    spec = {"base": 300.0, "dims": rot, "scaling": {"factor": 2.0}}
+    freq = np.array([300.0 ** (-2.0 * i / rot) / 2.0 for i in range(rot // 2)])
+    cos, sin = _f32(np.cos(pos[:, None] * freq)), _f32(np.sin(pos[:, None] * freq))
+    slots = rng.permutation(5 * page)[:T].astype(np.int32)
+    kc, vc = torch.zeros(5, nkv, page, dk, device=DEV), torch.zeros(5, nkv, page, dv, device=DEV)
+    d = _f32(qkv)
+    ops.qk_norm_pairs_store(d, nh, nkv, dk, dv, rot, _f32(wq), _f32(wk), 1e-5, cos, sin, torch.tensor(slots, device=DEV), kc, vc, page,
+                            half_split=True)
+    q = plain.rotate_half((plain.rms(qkv[:, :nh * dk], 1e-5) * wq).reshape(T, nh, dk), pos, spec)
+    k = plain.rotate_half((plain.rms(qkv[:, nh * dk:nh * dk + nkv * dk], 1e-5) * wk).reshape(T, nkv, dk), pos, spec)
+    v = qkv[:, nh * dk + nkv * dk:nh * dk + nkv * (dk + dv)].reshape(T, nkv, dv)
+    assert np.abs(d[:, :nh * dk].cpu().numpy().reshape(T, nh, dk) - q).max() < 1e-5
+    for t in range(T):
+        assert np.abs(kc[slots[t] // page, :, slots[t] % page].cpu().numpy() - k[t]).max() < 1e-5
+        assert np.abs(vc[slots[t] // page, :, slots[t] % page].cpu().numpy() - v[t]).max() < 1e-6
+
+
+def _sink_attention_case(dtype, seg_specs, nh, nkv, dk, dv, page, seed, heads_kernel=None):
+    """Random queries, keys and values for segments (context, queries) in shuffled pages, a sink a head and a gate a
+    (token, head); returns the kernel's output and softmax-with-sink by hand."""
+    from litinfer_amd.engine.batch import AttentionMeta
+    from litinfer_amd.engine.workspace import Workspace
+    from litinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(seed)
+    blocks = [-(-c // page) for c, _ in seg_specs]
+    num_pages = sum(blocks) + 2
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    kc, vc = torch.randn(num_pages, nkv, page, dk, generator=g).to(dtype), torch.randn(num_pages, nkv, page, dv, generator=g).to(dtype)
+    tab = np.full((len(seg_specs), max(blocks)), -1, dtype=np.int32)
+    T = sum(q for _, q in seg_specs)
+    q = torch.randn(T, nh, dk, generator=g)
+    sink = torch.randn(nh, generator=g) * 2.0
+    gate = torch.randn(T, nh + 3, generator=g)                               # (a view of columns inside wider rows)
+    scale = 1.0 / math.sqrt(dk)
+    refs, o, rep = [], 0, nh // nkv
+    for s, (c, ql) in enumerate(seg_specs):
+        k, v = torch.randn(c, nkv, dk, generator=g).to(dtype), torch.randn(c, nkv, dv, generator=g).to(dtype)
+        for b in range(blocks[s]):
+            tab[s, b] = perm.pop()
+            n = min(page, c - b * page)
+            kc[tab[s, b], :, :n] = k[b * page:b * page + n].transpose(0, 1)
+            vc[tab[s, b], :, :n] = v[b * page:b * page + n].transpose(0, 1)
+        kk, vv = k.double().numpy(), v.double().numpy()
+        out = np.zeros((ql, nh, dv))
+        for i in range(ql):
+            p = c - ql + i
+            for h in range(nh):
+                sc = kk[:p + 1, h // rep] @ q[o + i, h].double().numpy() * scale
+                mx = max(sc.max(), float(sink[h]))
+                e = np.exp(sc - mx)
+                out[i, h] = (e @ vv[:p + 1, h // rep]) / (e.sum() + math.exp(float(sink[h]) - mx)) / (1.0 + math.exp(-float(gate[o + i, 1 + h])))
+        refs.append(out.reshape(ql, -1))
+        o += ql
+    q_len = np.array([x for _, x in seg_specs], dtype=np.int32)
+    ctx_len = np.array([c for c, _ in seg_specs], dtype=np.int32)
+    q_start = np.concatenate([[0], np.cumsum(q_len)[:-1]]).astype(np.int32)
+    seg_of = np.repeat(np.arange(len(seg_specs), dtype=np.int32), q_len)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    single, multi = np.nonzero(q_len[seg_of] == 1)[0].astype(np.int32), np.nonzero(q_len[seg_of] != 1)[0].astype(np.int32)
+    tiles = np.asarray([(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0) for i in range(len(seg_specs))
+                        if q_len[i] > 1 for a in range(0, int(q_len[i]), 32)], dtype=np.int32).reshape(-1, 4)
+    meta = AttentionMeta(block_table=dev(tab), max_blocks=tab.shape[1], seg_of_token=dev(seg_of), q_start=dev(q_start), q_len=dev(q_len),
+                         ctx_len=dev(ctx_len), num_segments=len(seg_specs), num_tokens=T, max_q_len=int(q_len.max()),
+                         max_ctx_len=int(ctx_len.max()), host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len,
+                         single_tokens=dev(single) if len(multi) else None, num_single=len(single),
+                         multi_tokens=dev(multi) if len(single) else None, num_multi=len(multi),
+                         tiles=dev(tiles), num_tiles=len(tiles), tile_rows=32)
+    out = torch.empty(T, nh * dv, dtype=dtype, device=DEV)
+    gd = gate.to(DEV)
+    was = ops._heads_kernel_pays
+    if heads_kernel is not None:
+        ops._heads_kernel_pays = lambda *a: bool(heads_kernel)
+    try:
+        ops.masked_attention(q.to(DEV).contiguous(), nh * dk, dk, out, kc.to(DEV), vc.to(DEV), meta, nh, nkv, dk, dv, page, 0, 0, 0.0,
+                             scale, ws=Workspace(DEV), sink=sink.to(DEV), head_gate=gd[:, 1:1 + nh])
+    finally:
+        ops._heads_kernel_pays = was
+    return out.float().cpu().numpy(), np.concatenate(refs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("segs,nh,nkv,dk,dv,page,heads_kernel", [
+    ([(2, 2)], 1, 1, 4, 4, 16, None),                                          # the general kernel, one wave
+    ([(100, 37), (33, 2), (300, 1), (70, 70)], 6, 3, 24, 40, 8, None),         # ... four and eight waves a (token, head)
+    ([(700, 3), (5, 5)], 2, 1, 24, 16, 16, None),
+    ([(100, 37), (33, 2), (300, 1), (70, 70), (64, 64), (1, 1)], 6, 3, 64, 64, 8, None),   # tiles of queries beside single tokens
+    ([(1500, 1500)], 8, 2, 64, 64, 16, None),                                  # one long prompt: tiles whose keys are cut into splits
+    ([(900, 1), (90, 1), (3, 1), (2500, 1)], 8, 4, 64, 64, 16, False),         # single tokens, rows over lanes, splits and their join
+    ([(900, 1), (90, 1), (3, 1), (2500, 1)], 8, 2, 128, 128, 16, True),        # single tokens with the heads as a tile's columns
+    ([(40, 1)], 4, 4, 128, 64, 8, False),                                      # no splits: the finishing step inside the kernel
+    ([(40, 1)], 32, 1, 64, 64, 8, True),
+])
+def test_softmax_with_a_sink_and_a_gate_in_every_attention_kernel(dtype, segs, nh, nkv, dk, dv, page, heads_kernel):
+    got, ref = _sink_attention_case(dtype, segs, nh, nkv, dk, dv, page, seed=dk + nh, heads_kernel=heads_kernel)
+    err = float(np.abs(got - ref).max() / np.abs(ref).max())
+    assert err < (2e-5 if dtype is torch.float32 else 1.2e-2), err
+
+
+@pytest.mark.parametrize("E,ident,top,groups,keep", [(6, 2, 2, 4, 2), (12, 4, 3, 4, 3), (3, 0, 3, 1, 1), (4, 1, 1, 5, 5), (1, 1, 1, 1, 1),
+                                                   (60, 4, 6, 8, 3), (2, 6, 4, 2, 1)])
+def test_router_over_all_outputs_with_groups_scored_by_their_maximum(E, ident, top, groups, keep):
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(E)
+    T, K, n = 50, 40, E + ident
+    h, wr, corr = rng.normal(size=(T, K)), rng.normal(0, 0.4, size=(n, K)), rng.normal(0, 0.1, n)
+    idx, wt = torch.empty(T, top, dtype=torch.int32, device=DEV), torch.empty(T, top, device=DEV)
+    ops.moe_route(_f32(h), _f32(wr), None, None, idx, wt, None, scores="softmax", correction=_f32(corr), groups=groups, keep_groups=keep,
+                  group_score="max", normalize=False)
+    margins = []
+    want_i, want_w = plain.route(h, {"r.router": wr, "r.correction": corr}, "r.", {"experts": E, "identity": ident, "top": top,
+                                                                                  "groups": {"count": groups, "keep": keep}}, margins)
+    clear = margins[0] > 1e-5
+    assert clear.sum() > T // 2
+    assert np.array_equal(idx.cpu().numpy()[clear], want_i[clear])
+    assert np.abs(wt.cpu().numpy()[clear] - want_w[clear]).max() < 1e-6
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,K,E,ident,top,ff,groups,keep,limit", [(1, 96, 6, 2, 2, 40, 4, 2, 1.5), (70, 128, 12, 4, 3, 64, 4, 3, 2.0),
+                                                                   (300, 64, 3, 0, 3, 48, 1, 1, 7.0), (9, 256, 4, 1, 1, 72, 5, 5, 0.5),
+                                                                   (2500, 128, 8, 8, 4, 96, 4, 2, 2.0), (33, 48, 1, 3, 2, 16, 2, 2, 1.0)])
+def test_routed_feed_forward_with_identity_experts_and_the_clamped_activation(dt, T, K, E, ident, top, ff, groups, keep, limit):
+    """The routed part as a whole, through every product kernel (few rows, tiles of 32, tiles through LDS), on tokens whose
+    choice is no close call."""
+    from litinfer_amd.config import PartSpec
+    from litinfer_amd.engine.workspace import Workspace
+    from litinfer_amd.parts import BranchStream, Runtime, build_part
+    rng = np.random.default_rng(T + K)
+    mlp = {"router": {"experts": E, "identity": ident, "top": top, "groups": {"count": groups, "keep": keep}}, "expert": {"ff": ff, "limit": limit}}
+    W = {"m.router": rng.normal(0, 2.0 / math.sqrt(K), (E + ident, K)), "m.correction": rng.normal(0, 0.1, E + ident)}
+    for e in range(E):
+        W[f"m.e{e}.gate"], W[f"m.e{e}.up"] = rng.normal(0, 2.0 / math.sqrt(K), (ff, K)), rng.normal(0, 2.0 / math.sqrt(K), (ff, K))
+        W[f"m.e{e}.down"] = rng.normal(0, 1.0 / math.sqrt(ff), (K, ff))
+    W = {n: torch.tensor(a, dtype=torch.float32).to(DT[dt]) for n, a in W.items()}
+    h = torch.tensor(rng.normal(size=(T, K)), dtype=torch.float32).to(DT[dt])
+    part = build_part("feed_forward", PartSpec("routed_mlp", "m.", {
+        "hidden_size": K, "intermediate_size": ff, "experts": E, "identity": ident, "top": top, "activation": "clamped_swiglu",
+        "limit": limit, "scores": "softmax", "correction": True, "router_bias": False, "groups": groups, "keep_groups": keep,
+        "group_score": "max", "normalize": False}), Runtime(torch.device(DEV), DT[dt]))
+    part.load_params(lambda n: W.get(n))
+    ws = Workspace(DEV)
+    branch = BranchStream(torch.empty(T, K, device=DEV), ws)
+    part.forward(h.to(DEV), branch, SimpleNamespace(ws=ws))
+    W64 = {n: a.double().numpy() for n, a in W.items()}
+    margins = []
+    want = plain.moe_ff(h.double().numpy(), W64, "m.", mlp, margins)
+    clear = margins[0] > (1e-5 if dt == "float32" else 2e-2)
+    assert clear.sum() > T // 3 or T == 1
+    got = branch.result().cpu().numpy()
+    err = np.abs(got - want).max(axis=-1)[clear] / np.abs(want).max()
+    assert err.max() < (2e-5 if dt == "float32" else 2e-2), err.max()
