@@ -793,6 +793,32 @@ def tovasun_latent_config(size: str, layers: int, vocab: int = 32000) -> Dict[st
             "loop": {"start": 1, "stop": 3, "times": 2} if layers >= 4 else None}
 
 
+KUFOLORN_SIZES = {        # delta heads, their q/k heads; attention heads, kv heads; retention heads; key and value size of all three;
+    # experts, identity outputs, chosen, groups, kept groups, expert width (four chosen experts are as wide as the dense feed-forward)
+    "1.5b": (12, 6, 12, 2, 4, 128, 12, 4, 4, 4, 3, 2240),
+    "7b": (28, 14, 28, 4, 8, 128, 12, 4, 4, 4, 3, 4736),
+}
+
+
+def kufolorn_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, object]:
+    """A Kufolorn model at the width of a Qwen2 family member: gated delta-rule layers with every third one softmax
+    attention (sink, head gate, no window) beside a retention, a dense and a routed feed-forward in turn."""
+    width, ff = DESIGN_SIZES[size][0], DESIGN_SIZES[size][4]
+    dh, dkv, ah, akv, rh, dim, ne, ident, top, groups, keep, eff = KUFOLORN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0},
+           "router": {"experts": ne, "identity": ident, "top": top, "groups": {"count": groups, "keep": keep}}}
+    delta = {"heads": dh, "kv_heads": dkv, "dim": dim, "vdim": dim, "conv": 4}
+    par = {"left": {"heads": ah, "kv_heads": akv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                    "rot": {"base": 1000000.0, "dims": dim // 2, "scaling": {"factor": 2.0}}},
+           "right": {"heads": rh, "dim": dim, "vdim": dim, "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(rh)],
+                     "rot": {"base": 1000000.0, "dims": dim // 2}},
+           "left_scale": 0.6, "right_scale": 0.5}
+    return {"architecture": "Kufolorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": [{"type": "parallel" if i % 3 == 1 else "delta", "mixer": par if i % 3 == 1 else delta,
+                        "mlp": dense if i % 2 == 0 else moe} for i in range(layers)]}
+
+
 def compare_designs(a) -> Dict[str, object]:
     """Prefill and decode throughput of a second design (`--design`: Tovasun, Sogenex or Nusuvik) beside Qwen2 (Nusuvik:
     beside its closest relative, an all-latent Tovasun model) at the same width, heads, (active) feed-forward width,
@@ -807,19 +833,23 @@ def compare_designs(a) -> Dict[str, object]:
     for size in sizes:
         layers = a.layers or 6
         design = getattr(a, "design", None) or "tovasun"
-        tcfg = {"sogenex": sogenex_config, "nusuvik": nusuvik_config}.get(design, tovasun_config)(size, layers)
+        tcfg = {"sogenex": sogenex_config, "nusuvik": nusuvik_config, "kufolorn": kufolorn_config}.get(design, tovasun_config)(size, layers)
         runs = layers + (2 if tcfg.get("loop") else 0)
         width, heads, kv, dim, ff = DESIGN_SIZES[size][:5]
         if design == "nusuvik":
             beside, qcfg = "tovasun", tovasun_latent_config(size, layers)
+        elif design == "kufolorn":                   # its closest relative: recurrent layers, every third one attention, routed feed-forwards
+            beside, qcfg = "sogenex", sogenex_config(size, layers)
         else:
             beside = "qwen2"
             qcfg = dict(SHAPES[size], num_hidden_layers=runs, vocab_size=32000, use_sliding_window=True,
                         sliding_window=DESIGN_WINDOW, max_window_layers=0, max_position_embeddings=8192)
         res = {}
         for name, cfg, vocab in ((design, tcfg, tcfg["vocab"]), (beside, qcfg, 32000)):
+            if a.only and name != a.only:
+                continue
             eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
-                                     num_pages=(64 * ((2 if design == "nusuvik" else 1) * DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE,
+                                     num_pages=(64 * ((2 if design in ("nusuvik", "kufolorn") else 1) * DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE,
                                      max_seqs=65)
             for g in eng.cache.groups:
                 for data in g.data.values():
@@ -866,15 +896,16 @@ def compare_designs(a) -> Dict[str, object]:
             log(f"{size} {name}: {r}")
             del eng
             torch.cuda.empty_cache()
-        res[f"{design}_over_{beside}"] = {k: round(res[design][k] / res[beside][k], 3)
-                                          for k in res[beside] if k.endswith("tok_s")}
+        if design in res and beside in res:
+            res[f"{design}_over_{beside}"] = {k: round(res[design][k] / res[beside][k], 3)
+                                              for k in res[beside] if k.endswith("tok_s")}
         out[size] = res
     first = out[sizes[0]]
     title = design.capitalize()
     return {"metric": f"decode tok/s ({title} at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, "
-                      + ("no window)" if design == "nusuvik" else f"window {DESIGN_WINDOW})"),
-            "value": first[design][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
-            "warmup": a.warmup, "ms_per_step": first[design][f"decode_b{a.batch}_ms"], "higher_is_better": True,
+                      + ("no window)" if design in ("nusuvik", "kufolorn") else f"window {DESIGN_WINDOW})"),
+            "value": first[a.only or design][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": first[a.only or design][f"decode_b{a.batch}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
             "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content",
             "config": {"model": f"{title} beside {beside.capitalize()} at equal layer sizes", "global_batch": a.batch,
@@ -894,8 +925,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep", "designs"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="sweep: the member of the family whose layer sizes are taken (7b); designs: 1.5b or 7b (both)")
-    ap.add_argument("--design", default="tovasun", choices=["tovasun", "sogenex", "nusuvik"],
-                    help="designs: the design that is set beside Qwen2")
+    ap.add_argument("--design", default="tovasun", choices=["tovasun", "sogenex", "nusuvik", "kufolorn"],
+                    help="designs: the design that is set beside Qwen2 (Nusuvik: beside an all-latent Tovasun; Kufolorn: beside Sogenex)")
+    ap.add_argument("--only", default=None, help="designs: run one of the two models only (its name)")
     ap.add_argument("--page-order-seed", type=int, default=0,
                     help="headline: the cache's pages are handed out in a shuffled order, as a pool that has served requests "
                          "does (negative: in the order of their numbers; a request's keys then lie in one piece, and "
