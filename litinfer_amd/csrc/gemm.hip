@@ -199,8 +199,10 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
         const bool ok = WHOLE || k0 + 4 * lkq < K;         // (K % 4 == 0: a 16-byte piece is inside the row or past its end)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            ga[h] = *reinterpret_cast<const floatx4*>(xa[h] + (ok ? k0 : 0));
-            gb[h] = *reinterpret_cast<const floatx4*>(wb[h] + (ok ? k0 : 0));
+            // (a piece past the row's end is replaced by the row's first one, which is always there: with K < 16 the
+            // thread's own k-quarter may lie past the end of the LAST row, that is, of the tensor)
+            ga[h] = *reinterpret_cast<const floatx4*>(xa[h] + (ok ? k0 : -4 * lkq));
+            gb[h] = *reinterpret_cast<const floatx4*>(wb[h] + (ok ? k0 : -4 * lkq));
             if constexpr (!WHOLE) { if (!ok) { ga[h] = floatx4{0.f, 0.f, 0.f, 0.f}; gb[h] = floatx4{0.f, 0.f, 0.f, 0.f}; } }
         }
     };

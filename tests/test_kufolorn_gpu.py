@@ -657,3 +657,17 @@ def test_routed_feed_forward_with_identity_experts_and_the_clamped_activation(dt
     got = branch.result().cpu().numpy()
     err = np.abs(got - want).max(axis=-1)[clear] / np.abs(want).max()
     assert err.max() < (2e-5 if dt == "float32" else 2e-2), err.max()
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 64, 8), (150, 96, 4), (130, 48, 12), (99, 64, 8), (300, 320, 8)])
+def test_float32_products_whose_rows_are_shorter_than_a_step_of_the_kernel(M, N, K):
+    """A retention of one head of 8 columns makes the output projection a product with K = 8: the many-rows float32 kernel
+    goes through K in steps of 16, and a thread whose quarter of the step lies past K must not read from there (for the
+    last row that is past the tensor's end)."""
+    from litinfer_amd.kernels import ops
+    rng = np.random.default_rng(M + K)
+    x, w, b = rng.normal(size=(M, K)), rng.normal(size=(N, K)), rng.normal(size=N)
+    out = torch.empty(M, N, device=DEV)
+    ops.linear(_f32(x), _f32(w), _f32(b), out, False)
+    want = x @ w.T + b
+    assert np.abs(out.cpu().numpy() - want).max() < 1e-5 * np.abs(want).max()
