@@ -555,13 +555,24 @@ extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_ra
 // in LDS DR_TB tokens at a time (normed there: sixteen lanes a token add the squares in a fixed order).
 // Rows of xkq: [v: heads x vdim | k: G x N | q: G x N]; rows of ba: [b: heads | a: heads].
 #define DR_TB 16
+//
+// A step's portion of a request is cut into chunks of Q tokens that run side by side, as the state-space recurrence's
+// are.  Here a token's step is S <- A_t S + beta_t k_t v_t^T with the MATRIX A_t = g_t (I - beta_t k_t k_t^T), so what a
+// chunk does to the state it starts from is a matrix P = A_last ... A_first beside the state S_own that the chunk alone
+// builds up from zero:
+//   MODE 1: S_own of every chunk but a request's last, and P: its column j is what the recurrence, fed v = 0, makes of
+//           the unit vector e_j, so P is N more columns of the same kernel (stored transposed: PT[j][n]);
+//   the carry kernel: the state with which every chunk begins, chunk after chunk: S_in(c + 1) = P_c S_in(c) + S_own(c);
+//   MODE 0: the recurrence itself from that state, with the outputs; the last chunk leaves the request's state.
+// A portion of at most Q tokens (a decoding step) is MODE 0 alone, from the request's state.
 
-template <int NR, int NS, int CW>
+template <int NR, int NS, int CW, int MODE>
 __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
     const float* __restrict__ xkq, long x_stride, const float* __restrict__ ba, long ba_stride,
     const float* __restrict__ dt_bias, const float* __restrict__ A_log, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
-    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, float q_scale) {
+    const int* __restrict__ chunk_seg, const int* __restrict__ chunk_idx, float* __restrict__ carry, float* __restrict__ pmat,
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q, float q_scale) {
     constexpr int NP = NR * NS, PW = 64 * CW / NS;
     extern __shared__ __align__(16) float lds[];
     float* sK = lds;                                   // [DR_TB][NP]
@@ -569,30 +580,44 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
     float* sX = sQ + DR_TB * NP;                       // [SSM_WAVES][DR_TB][PW]
     float* sBeta = sX + SSM_WAVES * DR_TB * PW;        // [SSM_WAVES][DR_TB]
     float* sG = sBeta + SSM_WAVES * DR_TB;             // [SSM_WAVES][DR_TB]
-    const int seg = blockIdx.x;
-    const int ntok = q_len[seg];
-    if (ntok <= 0) return;
-    const int t0 = q_start[seg];
-    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    const int bx = blockIdx.x;
+    const int seg = chunk_seg ? chunk_seg[bx] : bx;
+    if (seg < 0) return;
+    const int c = chunk_seg ? chunk_idx[bx] : 0;
+    const int L = q_len[seg], first = c * Q;
+    if (first >= L) return;
+    const int ntok = chunk_seg ? ((L - first < Q) ? L - first : Q) : L;
+    const bool last = first + ntok >= L;
+    if (MODE == 1 && last) return;                      // nobody needs the last chunk's own state
+    const int t0 = q_start[seg] + first;
+    // units of a head: blocks of PW value columns, and in MODE 1 behind them blocks of PW columns of P
+    const int hpg = heads / G, PSV = (vdim + PW - 1) / PW, PS = PSV + (MODE == 1 ? (N + PW - 1) / PW : 0);
+    const int U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
     const int g = blockIdx.y / ublocks, ub = blockIdx.y % ublocks;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int unit = ub * SSM_WAVES + w;
     const bool active = unit < U;
-    const int head = g * hpg + (active ? unit / PS : 0), pbase = active ? (unit % PS) * PW : 0;
+    const int head = g * hpg + (active ? unit / PS : 0), sub = active ? unit % PS : 0;
+    const bool is_p = MODE == 1 && sub >= PSV;
+    const int pbase = (is_p ? sub - PSV : sub) * PW, ncols = is_p ? N : vdim;
     const int pq = lane / NS, s = lane % NS, p = pbase + CW * pq;       // the first of the lane's columns
     const int inner = heads * vdim;
     float* st = state + ((size_t)slots[seg] * heads + head) * N * vdim;
+    const float* src = chunk_seg ? carry + ((size_t)bx * heads + head) * N * vdim : st;
     float S[NR][CW];
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
         const int n = s * NR + r;
-        if constexpr (CW == 4) {
-            const float4 v4 = (active && n < N && p < vdim) ? *reinterpret_cast<const float4*>(st + (size_t)n * vdim + p)
+        if (MODE == 1) {
+#pragma unroll
+            for (int cc = 0; cc < CW; ++cc) S[r][cc] = (is_p && n == p + cc) ? 1.f : 0.f;
+        } else if constexpr (CW == 4) {
+            const float4 v4 = (active && n < N && p < vdim) ? *reinterpret_cast<const float4*>(src + (size_t)n * vdim + p)
                                                             : float4{0.f, 0.f, 0.f, 0.f};
             S[r][0] = v4.x; S[r][1] = v4.y; S[r][2] = v4.z; S[r][3] = v4.w;
         } else {
 #pragma unroll
-            for (int c = 0; c < CW; ++c) S[r][c] = (active && n < N && p + c < vdim) ? st[(size_t)n * vdim + p + c] : 0.f;
+            for (int cc = 0; cc < CW; ++cc) S[r][cc] = (active && n < N && p + cc < vdim) ? src[(size_t)n * vdim + p + cc] : 0.f;
         }
     }
     for (int b0 = 0; b0 < ntok; b0 += DR_TB) {
@@ -607,12 +632,12 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
         if (active) {
             for (int i = lane; i < DR_TB * PW; i += 64) {
                 const int tt = i / PW, pp = pbase + i % PW;
-                const bool ok = b0 + tt < ntok && pp < vdim;
+                const bool ok = !is_p && b0 + tt < ntok && pp < vdim;
                 sX[(w * DR_TB + tt) * PW + i % PW] = ok ? xkq[(size_t)(t0 + b0 + tt) * x_stride + (size_t)head * vdim + pp] : 0.f;
             }
             if (lane < DR_TB) {
                 const bool ok = b0 + lane < ntok;
-                const float* r2 = ba + (size_t)(t0 + b0 + lane) * ba_stride;
+                const float* r2 = ba + (size_t)(t0 + b0 + (ok ? lane : 0)) * ba_stride;
                 sBeta[w * DR_TB + lane] = ok ? 1.0f / (1.0f + expf(-r2[head])) : 0.f;
                 sG[w * DR_TB + lane] = ok ? expf(-expf(A_log[head]) * softplus_f32(r2[heads + head] + dt_bias[head])) : 1.f;
             }
@@ -644,12 +669,12 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
             const float gd = sG[w * DR_TB + tt], beta = sBeta[w * DR_TB + tt];
             float xv[CW];
 #pragma unroll
-            for (int c = 0; c < CW; ++c) xv[c] = sX[(w * DR_TB + tt) * PW + CW * pq + c];
+            for (int cc = 0; cc < CW; ++cc) xv[cc] = sX[(w * DR_TB + tt) * PW + CW * pq + cc];
             const float4* Kp = reinterpret_cast<const float4*>(sK + tt * NP + s * NR);
             const float4* Qp = reinterpret_cast<const float4*>(sQ + tt * NP + s * NR);
             float ks[CW];
 #pragma unroll
-            for (int c = 0; c < CW; ++c) ks[c] = 0.f;
+            for (int cc = 0; cc < CW; ++cc) ks[cc] = 0.f;
 #pragma unroll
             for (int r4 = 0; r4 < NR / 4; ++r4) {
                 const float4 kv = Kp[r4];
@@ -657,81 +682,186 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) ks[c] = fmaf(S[4 * r4 + j][c], kk[j], ks[c]);
+                    for (int cc = 0; cc < CW; ++cc) ks[cc] = fmaf(S[4 * r4 + j][cc], kk[j], ks[cc]);
             }
 #pragma unroll
             for (int o = 1; o < NS; o <<= 1)
 #pragma unroll
-                for (int c = 0; c < CW; ++c) ks[c] += __shfl_xor(ks[c], o, LI_WAVE);
+                for (int cc = 0; cc < CW; ++cc) ks[cc] += __shfl_xor(ks[cc], o, LI_WAVE);
             float u[CW], ov[CW];
 #pragma unroll
-            for (int c = 0; c < CW; ++c) { u[c] = beta * (xv[c] - gd * ks[c]); ov[c] = 0.f; }
+            for (int cc = 0; cc < CW; ++cc) { u[cc] = beta * (xv[cc] - gd * ks[cc]); ov[cc] = 0.f; }
 #pragma unroll
             for (int r4 = 0; r4 < NR / 4; ++r4) {
-                const float4 qv = Qp[r4], kv = Kp[r4];
-                const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, kk[4] = {kv.x, kv.y, kv.z, kv.w};
+                const float4 kv = Kp[r4];
+                const float kk[4] = {kv.x, kv.y, kv.z, kv.w};
+                float qs[4] = {0.f, 0.f, 0.f, 0.f};
+                if (MODE == 0) { const float4 qv = Qp[r4]; qs[0] = qv.x; qs[1] = qv.y; qs[2] = qv.z; qs[3] = qv.w; }
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) {
-                        const float nv = fmaf(gd, S[4 * r4 + j][c], kk[j] * u[c]);
-                        S[4 * r4 + j][c] = nv;
-                        ov[c] = fmaf(nv, qs[j], ov[c]);
+                    for (int cc = 0; cc < CW; ++cc) {
+                        const float nv = fmaf(gd, S[4 * r4 + j][cc], kk[j] * u[cc]);
+                        S[4 * r4 + j][cc] = nv;
+                        if (MODE == 0) ov[cc] = fmaf(nv, qs[j], ov[cc]);
                     }
             }
+            if (MODE == 0) {
 #pragma unroll
-            for (int o = 1; o < NS; o <<= 1)
+                for (int o = 1; o < NS; o <<= 1)
 #pragma unroll
-                for (int c = 0; c < CW; ++c) ov[c] += __shfl_xor(ov[c], o, LI_WAVE);
-            if (s == 0) {
-                float* yr = y + (size_t)(t0 + b0 + tt) * y_stride + (size_t)head * vdim + p;
-                if constexpr (CW == 4) {
-                    if (p < vdim) *reinterpret_cast<float4*>(yr) = float4{ov[0], ov[1], ov[2], ov[3]};
-                } else {
+                    for (int cc = 0; cc < CW; ++cc) ov[cc] += __shfl_xor(ov[cc], o, LI_WAVE);
+                if (s == 0) {
+                    float* yr = y + (size_t)(t0 + b0 + tt) * y_stride + (size_t)head * vdim + p;
+                    if constexpr (CW == 4) {
+                        if (p < vdim) *reinterpret_cast<float4*>(yr) = float4{ov[0], ov[1], ov[2], ov[3]};
+                    } else {
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) if (p + c < vdim) yr[c] = ov[c];
+                        for (int cc = 0; cc < CW; ++cc) if (p + cc < vdim) yr[cc] = ov[cc];
+                    }
                 }
             }
         }
     }
     if (!active) return;
+    if (MODE == 1 && is_p) {                            // PT[j][n]: the lane's columns j, its n values side by side
+        float* pt = pmat + ((size_t)bx * heads + head) * N * N;
+#pragma unroll
+        for (int cc = 0; cc < CW; ++cc)
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                const int n = s * NR + r;
+                if (n < N && p + cc < N) pt[(size_t)(p + cc) * N + n] = S[r][cc];
+            }
+        return;
+    }
+    float* dst = MODE == 1 ? carry + ((size_t)bx * heads + head) * N * vdim : (last ? st : nullptr);
+    if (!dst) return;
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
         const int n = s * NR + r;
         if (n >= N) continue;
         if constexpr (CW == 4) {
-            if (p < vdim) *reinterpret_cast<float4*>(st + (size_t)n * vdim + p) = float4{S[r][0], S[r][1], S[r][2], S[r][3]};
+            if (p < vdim) *reinterpret_cast<float4*>(dst + (size_t)n * vdim + p) = float4{S[r][0], S[r][1], S[r][2], S[r][3]};
         } else {
 #pragma unroll
-            for (int c = 0; c < CW; ++c) if (p + c < vdim) st[(size_t)n * vdim + p + c] = S[r][c];
+            for (int cc = 0; cc < CW; ++cc) if (p + cc < vdim) dst[(size_t)n * vdim + p + cc] = S[r][cc];
         }
+    }
+    (void)ncols;
+}
+
+// carry[chunk] holds what the chunk alone built up from zero, pmat[chunk] its matrix (transposed); afterwards carry[chunk]
+// holds the state with which the chunk begins.  A block takes a request, a head and DC_COLS columns of the state, chunk
+// after chunk; the state's columns lie in LDS, thread (slice, column) owns N / DC_SLICES values of the column.
+#define DC_COLS 16
+#define DC_SLICES 16
+#define DC_MAX 16                   // N / DC_SLICES at most: N <= 256
+__global__ __launch_bounds__(DC_COLS * DC_SLICES) void delta_carry_kernel(
+    float* __restrict__ carry, const float* __restrict__ pmat, const float* __restrict__ state, const int* __restrict__ slots,
+    const int* __restrict__ q_len, const int* __restrict__ chunk_first, int heads, int vdim, int N, int Q) {
+    extern __shared__ float run[];                      // [N][DC_COLS + 1]
+    const int seg = blockIdx.x, head = blockIdx.y, col = blockIdx.z * DC_COLS + (threadIdx.x % DC_COLS), sl = threadIdx.x / DC_COLS;
+    const int cl = threadIdx.x % DC_COLS;
+    const int nch = (q_len[seg] + Q - 1) / Q, base = chunk_first[seg];
+    const int per = (N + DC_SLICES - 1) / DC_SLICES, n0 = sl * per;
+    const bool on = col < vdim;
+    const float* stp = state + ((size_t)slots[seg] * heads + head) * N * vdim;
+    for (int i = 0; i < per; ++i)
+        if (n0 + i < N) run[(n0 + i) * (DC_COLS + 1) + cl] = on ? stp[(size_t)(n0 + i) * vdim + col] : 0.f;
+    __syncthreads();
+    for (int k = 0; k < nch; ++k) {
+        float* at = carry + ((size_t)(base + k) * heads + head) * N * vdim;
+        const float* pt = pmat + ((size_t)(base + k) * heads + head) * N * N;
+        float acc[DC_MAX];
+        const bool more = k + 1 < nch;
+#pragma unroll
+        for (int i = 0; i < DC_MAX; ++i) acc[i] = (more && on && i < per && n0 + i < N) ? at[(size_t)(n0 + i) * vdim + col] : 0.f;
+        if (more) {
+            for (int j = 0; j < N; ++j) {
+                const float cv = run[j * (DC_COLS + 1) + cl];
+                const float* prow = pt + (size_t)j * N + n0;
+#pragma unroll
+                for (int i = 0; i < DC_MAX; ++i)
+                    if (i < per && n0 + i < N) acc[i] = fmaf(prow[i], cv, acc[i]);
+            }
+        }
+        // the chunk begins with `run`; the next one with what has just been added up
+#pragma unroll
+        for (int i = 0; i < DC_MAX; ++i)
+            if (on && i < per && n0 + i < N) at[(size_t)(n0 + i) * vdim + col] = run[(n0 + i) * (DC_COLS + 1) + cl];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < DC_MAX; ++i)
+            if (i < per && n0 + i < N) run[(n0 + i) * (DC_COLS + 1) + cl] = acc[i];
+        __syncthreads();
     }
 }
 
 template <int NR, int NS, int CW>
 static int delta_launch(const float* xkq, long x_stride, const float* ba, long ba_stride, const float* dt_bias, const float* A_log,
-                        float* state, const int* slots, const int* q_start, const int* q_len, float* y, long y_stride,
-                        int heads, int vdim, int N, int G, float q_scale, int segs, hipStream_t stream) {
+                        float* state, const int* slots, const int* q_start, const int* q_len, int* chunk_tab, float* carry,
+                        float* pmat, float* y, long y_stride, int heads, int vdim, int N, int G, int Q, float q_scale, int segs,
+                        int max_chunks, bool chunked, hipStream_t stream) {
     constexpr int NP = NR * NS, PW = 64 * CW / NS;
     const size_t lds = (size_t)(2 * DR_TB * NP + SSM_WAVES * DR_TB * PW + 2 * SSM_WAVES * DR_TB) * sizeof(float);
-    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
-    delta_scan_kernel<NR, NS, CW><<<dim3(segs, G * ublocks), 64 * SSM_WAVES, lds, stream>>>(
-        xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, y, y_stride, heads, vdim, N, G, q_scale);
+    const int hpg = heads / G, PSV = (vdim + PW - 1) / PW, PSP = (N + PW - 1) / PW;
+    const int ub0 = (hpg * PSV + SSM_WAVES - 1) / SSM_WAVES, ub1 = (hpg * (PSV + PSP) + SSM_WAVES - 1) / SSM_WAVES;
+    if (!chunked) {
+        delta_scan_kernel<NR, NS, CW, 0><<<dim3(segs, G * ub0), 64 * SSM_WAVES, lds, stream>>>(
+            xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, nullptr, nullptr, nullptr, nullptr,
+            y, y_stride, heads, vdim, N, G, Q, q_scale);
+        return li_launch_status();
+    }
+    int* chunk_seg = chunk_tab;
+    int* chunk_idx = chunk_tab + max_chunks;
+    int* chunk_first = chunk_tab + 2 * max_chunks;
+    ssm_chunk_index_kernel<<<1, 256, 0, stream>>>(q_len, segs, Q, max_chunks, chunk_seg, chunk_idx, chunk_first);
+    delta_scan_kernel<NR, NS, CW, 1><<<dim3(max_chunks, G * ub1), 64 * SSM_WAVES, lds, stream>>>(
+        xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, pmat,
+        y, y_stride, heads, vdim, N, G, Q, q_scale);
+    delta_carry_kernel<<<dim3(segs, heads, (vdim + DC_COLS - 1) / DC_COLS), DC_COLS * DC_SLICES,
+                         (size_t)N * (DC_COLS + 1) * sizeof(float), stream>>>(carry, pmat, state, slots, q_len, chunk_first, heads, vdim, N, Q);
+    delta_scan_kernel<NR, NS, CW, 0><<<dim3(max_chunks, G * ub0), 64 * SSM_WAVES, lds, stream>>>(
+        xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, pmat,
+        y, y_stride, heads, vdim, N, G, Q, q_scale);
     return li_launch_status();
 }
 
 // 1 if the recurrence has a layout for a state of N values a column (the state-space recurrence's layouts)
 extern "C" int li_delta_scan_takes(int N, int vdim) { return li_ssm_scan_layout(N, vdim, nullptr, nullptr); }
 
+// Chunks that a step of T tokens in `segs` portions can have at most, and the bytes of the tables, states and matrices
+// that the chunked form keeps in the workspace.
+extern "C" long li_delta_scan_work_bytes(int T, int segs, int heads, int vdim, int N, int Q, int* max_chunks) {
+    const long mc = (long)T / Q + segs;
+    if (max_chunks) *max_chunks = (int)mc;
+    const long ints = ((3 * mc + segs + 1 + 3) / 4) * 4;
+    return ints * 4 + mc * heads * ((long)N * vdim + (long)N * N) * 4;
+}
+
 extern "C" int li_delta_scan(const float* xkq, long x_stride, const float* ba, long ba_stride, const float* dt_bias,
                              const float* A_log, float* state, const int* slots, const int* q_start, const int* q_len,
-                             float* y, long y_stride, int heads, int vdim, int N, int G, float q_scale, int T, int segs,
-                             hipStream_t stream) {
-    if (T <= 0 || segs <= 0 || heads <= 0 || G <= 0 || heads % G || vdim <= 0 || N <= 0 ||
+                             float* y, long y_stride, int heads, int vdim, int N, int G, float q_scale, int Q, int T, int segs,
+                             int max_q_len, void* work, long work_bytes, hipStream_t stream) {
+    if (T <= 0 || segs <= 0 || heads <= 0 || G <= 0 || heads % G || vdim <= 0 || N <= 0 || N > 256 || Q <= 0 || max_q_len <= 0 ||
         x_stride < (long)heads * vdim + 2L * G * N || ba_stride < 2L * heads || y_stride < (long)heads * vdim)
         return LI_ERR_SIZE;
-#define DR_ARGS xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, y, y_stride, heads, vdim, N, G, q_scale, segs, stream
-    const bool aligned = ((uintptr_t)state | (uintptr_t)y) % 16 == 0 && y_stride % 4 == 0;
+    const bool chunked = max_q_len > Q;
+    int max_chunks = 0;
+    int* chunk_tab = nullptr;
+    float *carry = nullptr, *pmat = nullptr;
+    if (chunked) {
+        const long need = li_delta_scan_work_bytes(T, segs, heads, vdim, N, Q, &max_chunks);
+        if (!work || work_bytes < need || ((uintptr_t)work % 16)) return LI_ERR_SIZE;
+        chunk_tab = (int*)work;
+        const long ints = ((3L * max_chunks + segs + 1 + 3) / 4) * 4;
+        carry = (float*)work + ints;
+        pmat = carry + (size_t)max_chunks * heads * N * vdim;
+    }
+#define DR_ARGS xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, chunk_tab, carry, pmat, y, y_stride, heads, \
+                vdim, N, G, Q, q_scale, segs, max_chunks, chunked, stream
+    const bool aligned = ((uintptr_t)state | (uintptr_t)y | (uintptr_t)carry) % 16 == 0 && y_stride % 4 == 0;
     int qs = 0, qr = 0;
     if (aligned && ssm_quad_layout(N, vdim, &qs, &qr)) {
 #define DR_QUAD(NR_, NS_) if (qr == NR_ && qs == NS_) return delta_launch<NR_, NS_, 4>(DR_ARGS);

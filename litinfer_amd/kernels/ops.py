@@ -57,7 +57,7 @@ _SIGNATURES = {
     "recurrent": {
         "li_causal_conv_silu": [P, L, I, I, P, P, P, P, P, P, P, P, L, I, I, I],
         "li_ssm_scan": [P, L, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, L, P, F],
-        "li_delta_scan": [P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, F, I, I],
+        "li_delta_scan": [P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, F, I, I, I, I, P, L],
         "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I, I],
     },
     "moe": {
@@ -1552,18 +1552,25 @@ def ssm_scan(xbc: torch.Tensor, dt: Optional[torch.Tensor], dt_bias: Optional[to
          ptr(fixed_decay), float(fixed_step))
 
 
+# Portions of more than SSM_CHUNK tokens run through the delta rule as chunks side by side (their own states and transition
+# matrices, the carry, the outputs); False: token after token, whatever the portion.
+DELTA_CHUNKED = True
+
+
 def delta_scan_takes(n_state: int, vdim: int) -> bool:
     """Whether the delta-rule kernel has a layout for states of `n_state` values a column."""
     return bool(_lib_fn("recurrent", "li_delta_scan_takes", [c_int, c_int], c_int)(int(n_state), int(vdim)))
 
 
 def delta_scan(xkq: torch.Tensor, ba: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, ctx,
-               y: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, q_scale: float) -> None:
+               y: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, q_scale: float, ws=None) -> None:
     """The gated delta rule over each request's tokens of the step, from and into `state` [slots, heads, n_state, vdim]
     (float32):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  y = S^T q,  with k and q made unit vectors
     (x / sqrt(sum x^2 + 1e-6); q times q_scale), beta = sigmoid(b), g = exp(-exp(a_log_h) softplus(a + dt_bias_h)).
     xkq: float32 rows [v: heads * vdim | k: groups * n_state | q: groups * n_state]; ba: float32 rows [b: heads | a: heads]
-    (raw); y: float32 rows [heads * vdim].  All float32."""
+    (raw); y: float32 rows [heads * vdim].  All float32.  With a workspace `ws`, portions longer than SSM_CHUNK tokens run
+    as chunks side by side (every chunk's own state and its transition matrix, then the chunks' starting states one after
+    the other, then the outputs); without one, token after token."""
     _gpu(xkq, ba, dt_bias, a_log, state, y)
     t = y.shape[0]
     inner = heads * vdim
@@ -1574,10 +1581,22 @@ def delta_scan(xkq: torch.Tensor, ba: torch.Tensor, dt_bias: torch.Tensor, a_log
          and all(v.numel() == heads and v.is_contiguous() for v in (dt_bias, a_log)), "delta_scan: state [slots, heads, N, vdim]")
     _chk(ctx.num_tokens == t and int(ctx.host_state_slots.max(initial=0)) < state.shape[0], "delta_scan: batch")
     _chk(delta_scan_takes(n_state, vdim), f"delta_scan: no kernel for a state of {n_state} values a column (at most 256)")
-    if t:
-        _run("recurrent", "li_delta_scan", xkq.data_ptr(), xkq.stride(0), ba.data_ptr(), ba.stride(0), dt_bias.data_ptr(),
-             a_log.data_ptr(), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(),
-             y.data_ptr(), y.stride(0), heads, vdim, n_state, groups, float(q_scale), t, ctx.num_segments)
+    if not t:
+        return
+    work, work_bytes, q = 0, 0, SSM_CHUNK
+    if not DELTA_CHUNKED:
+        ws = None
+    if ctx.max_q_len > SSM_CHUNK and ws is not None:
+        need = _lib_fn("recurrent", "li_delta_scan_work_bytes", [c_int] * 6 + [c_void_p], c_long)(
+            t, ctx.num_segments, heads, vdim, n_state, SSM_CHUNK, None)
+        buf = ws.buffer("delta_scan.work", ((int(need) + 3) // 4,), torch.float32)
+        work, work_bytes = buf.data_ptr(), buf.numel() * 4
+    elif ctx.max_q_len > SSM_CHUNK:
+        q = int(ctx.max_q_len)                       # one chunk a request: the recurrence token after token
+    _run("recurrent", "li_delta_scan", xkq.data_ptr(), xkq.stride(0), ba.data_ptr(), ba.stride(0), dt_bias.data_ptr(),
+         a_log.data_ptr(), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(),
+         y.data_ptr(), y.stride(0), heads, vdim, n_state, groups, float(q_scale), q, t, ctx.num_segments, int(ctx.max_q_len),
+         work, work_bytes)
 
 
 def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int, out: torch.Tensor,

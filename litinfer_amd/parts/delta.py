@@ -93,7 +93,7 @@ class GatedDeltaMixer(Mixer):
         ops.causal_conv_silu(proj[:, inner:inner + self.channels], self.conv_w, None, tail, ctx, vkq)
         y = ctx.ws.buffer("delta.y", (t, inner), torch.float32)
         ops.delta_scan(vkq, proj[:, inner + self.channels:], self.dt_bias, self.a_log, state, ctx, y, self.heads, self.vdim,
-                       self.dim, self.groups, self.dim ** -0.5)
+                       self.dim, self.groups, self.dim ** -0.5, ws=ctx.ws)
         g = ctx.ws.buffer("delta.gated", (t, inner), self.rt.dtype)
         ops.gated_group_norm(y, proj[:, :inner], self.norm_w, self.eps, self.heads, g, gate_after=True)
         residual.add_linear(self.out, g)

@@ -404,9 +404,14 @@ STEPS = ([(0, 1), (2, 5)], [(2, 1), (0, 2)], [(0, 1)], [(0, 20), (2, 2)], [(2, 1
 
 @pytest.mark.parametrize("heads,groups,N,vdim", [(6, 3, 24, 16), (2, 2, 8, 40), (4, 2, 128, 64), (8, 8, 64, 32), (12, 3, 16, 20),
                                                  (1, 1, 256, 8), (2, 1, 32, 128), (3, 1, 100, 6), (2, 2, 128, 128)])
-def test_delta_rule_across_steps_and_slots(heads, groups, N, vdim):
-    """Two requests on slots 0 and 2 take turns with portions of 1 to 100 tokens; slot 1 is nobody's and stays as it is."""
+@pytest.mark.parametrize("chunked", [False, True])
+def test_delta_rule_across_steps_and_slots(heads, groups, N, vdim, chunked):
+    """Two requests on slots 0 and 2 take turns with portions of 1 to 100 tokens; slot 1 is nobody's and stays as it is.
+    `chunked`: portions of more than 64 tokens run as chunks side by side (their own states and transition matrices, the
+    carry, the outputs); else token after token."""
+    from litinfer_amd.engine.workspace import Workspace
     from litinfer_amd.kernels import ops
+    ws = Workspace(DEV)
     rng = np.random.default_rng(N + vdim)
     inner, rep = heads * vdim, heads // groups
     a_log, dt_bias = rng.uniform(-3, 0, heads), rng.normal(0, 0.5, heads)
@@ -429,7 +434,7 @@ def test_delta_rule_across_steps_and_slots(heads, groups, N, vdim):
         wide[:, 3:] = _f32(ba)
         y = torch.empty(len(x), inner, device=DEV)
         ops.delta_scan(_f32(x), wide[:, 3:], _f32(dt_bias), _f32(a_log), state, _ctx([n for _, n in step], [s for s, _ in step]),
-                       y, heads, vdim, N, groups, N ** -0.5)
+                       y, heads, vdim, N, groups, N ** -0.5, ws=ws if chunked else None)
         want = np.concatenate([ref[s][at[s]:at[s] + n] for s, n in step])
         assert np.abs(y.cpu().numpy() - want).max() < 2e-5 * max(1.0, np.abs(want).max()), step
         for s, n in step:
