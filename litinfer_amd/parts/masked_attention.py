@@ -101,12 +101,12 @@ class MaskedAttention(Mixer):
         ws = [get(p + n[x]) for x in "qkv"]
         if self.head_gate:                  # the gates' rows ride behind q, k and v in the one packed product
             g = get(p + n["gate"])         # (with rows of zeros up to a multiple of four, so that a token's row keeps 16-byte pieces)
-            ws.append(torch.cat([g, torch.zeros(self.gate_cols - self.nh, self.hidden, dtype=g.dtype)], dim=0))
+            ws.append(torch.cat([g, g.new_zeros(self.gate_cols - self.nh, self.hidden)], dim=0))
         dt = torch.float32 if any(w.dtype is torch.float32 for w in ws) else ws[0].dtype
         bias = None
         if self.bias:
-            bias = torch.cat([get(p + n[x] + n["bias_suffix"]).to(torch.float32) for x in "qkv"]
-                             + ([torch.zeros(self.gate_cols)] if self.head_gate else []))
+            bs = [get(p + n[x] + n["bias_suffix"]).to(torch.float32) for x in "qkv"]
+            bias = torch.cat(bs + ([bs[0].new_zeros(self.gate_cols)] if self.head_gate else []))
         self.qkv = Linear(self.rt, torch.cat([w.to(dt) for w in ws], dim=0), bias)
         self.out = Linear(self.rt, get(p + n["o"]))
         if self.has_sink:
