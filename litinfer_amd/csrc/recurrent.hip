@@ -753,49 +753,88 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void delta_scan_kernel(
 
 // carry[chunk] holds what the chunk alone built up from zero, pmat[chunk] its matrix (transposed); afterwards carry[chunk]
 // holds the state with which the chunk begins.  A block takes a request, a head and DC_COLS columns of the state, chunk
-// after chunk; the state's columns lie in LDS, thread (slice, column) owns N / DC_SLICES values of the column.
+// after chunk; the state's columns lie in LDS, thread (slice, column) owns PER consecutive values of the column
+// (DC_SLICES * PER >= N).  A chunk's step is a product P x (state's columns): the thread walks P's rows j, which hold its
+// PER values side by side, DC_AHEAD rows at a time: their loads are issued
+// together and without conditions (a value past N reads the row's last one and is never stored), so that a trip to memory
+// serves DC_AHEAD rows and not one.
 #define DC_COLS 16
 #define DC_SLICES 16
-#define DC_MAX 16                   // N / DC_SLICES at most: N <= 256
+#define DC_ROUND 16                 // the state's rows in LDS are rounded up to this: the most rows a trip takes
+template <int PER, int DC_AHEAD, bool VEC>      // VEC: N and PER multiples of 4, P on 16 bytes: a row's values in 16-byte pieces
 __global__ __launch_bounds__(DC_COLS * DC_SLICES) void delta_carry_kernel(
     float* __restrict__ carry, const float* __restrict__ pmat, const float* __restrict__ state, const int* __restrict__ slots,
     const int* __restrict__ q_len, const int* __restrict__ chunk_first, int heads, int vdim, int N, int Q) {
-    extern __shared__ float run[];                      // [N][DC_COLS + 1]
-    const int seg = blockIdx.x, head = blockIdx.y, col = blockIdx.z * DC_COLS + (threadIdx.x % DC_COLS), sl = threadIdx.x / DC_COLS;
-    const int cl = threadIdx.x % DC_COLS;
+    extern __shared__ float run[];                      // [N rounded up to DC_ROUND][DC_COLS + 1]
+    const int seg = blockIdx.x, head = blockIdx.y, cl = threadIdx.x % DC_COLS, sl = threadIdx.x / DC_COLS;
+    const int col = blockIdx.z * DC_COLS + cl;
     const int nch = (q_len[seg] + Q - 1) / Q, base = chunk_first[seg];
-    const int per = (N + DC_SLICES - 1) / DC_SLICES, n0 = sl * per;
+    const int n0 = sl * PER;
     const bool on = col < vdim;
+    const int NA = (N + DC_ROUND - 1) / DC_ROUND * DC_ROUND;
     const float* stp = state + ((size_t)slots[seg] * heads + head) * N * vdim;
-    for (int i = 0; i < per; ++i)
-        if (n0 + i < N) run[(n0 + i) * (DC_COLS + 1) + cl] = on ? stp[(size_t)(n0 + i) * vdim + col] : 0.f;
+    int off[PER];                                       // the thread's values within a row of P (clamped: loads carry no conditions)
+#pragma unroll
+    for (int i = 0; i < PER; ++i) off[i] = n0 + i < N ? n0 + i : N - 1;
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+        if (n0 + i < NA) run[(n0 + i) * (DC_COLS + 1) + cl] = (on && n0 + i < N) ? stp[(size_t)(n0 + i) * vdim + col] : 0.f;
     __syncthreads();
     for (int k = 0; k < nch; ++k) {
         float* at = carry + ((size_t)(base + k) * heads + head) * N * vdim;
         const float* pt = pmat + ((size_t)(base + k) * heads + head) * N * N;
-        float acc[DC_MAX];
+        float acc[PER];
         const bool more = k + 1 < nch;
 #pragma unroll
-        for (int i = 0; i < DC_MAX; ++i) acc[i] = (more && on && i < per && n0 + i < N) ? at[(size_t)(n0 + i) * vdim + col] : 0.f;
+        for (int i = 0; i < PER; ++i) acc[i] = (more && on && n0 + i < N) ? at[(size_t)(n0 + i) * vdim + col] : 0.f;
         if (more) {
-            for (int j = 0; j < N; ++j) {
-                const float cv = run[j * (DC_COLS + 1) + cl];
-                const float* prow = pt + (size_t)j * N + n0;
+            for (int j0 = 0; j0 < N; j0 += DC_AHEAD) {
+                float pv[DC_AHEAD][PER], cv[DC_AHEAD];
 #pragma unroll
-                for (int i = 0; i < DC_MAX; ++i)
-                    if (i < per && n0 + i < N) acc[i] = fmaf(prow[i], cv, acc[i]);
+                for (int u = 0; u < DC_AHEAD; ++u) {
+                    const float* prow = pt + (size_t)(j0 + u < N ? j0 + u : N - 1) * N;
+                    if constexpr (VEC) {
+#pragma unroll
+                        for (int v = 0; v < PER / 4; ++v) {
+                            const float4 t4 = *reinterpret_cast<const float4*>(prow + (n0 + 4 * v < N ? n0 + 4 * v : N - 4));
+                            pv[u][4 * v] = t4.x; pv[u][4 * v + 1] = t4.y; pv[u][4 * v + 2] = t4.z; pv[u][4 * v + 3] = t4.w;
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < PER; ++i) pv[u][i] = prow[off[i]];
+                    }
+                    cv[u] = run[(j0 + u) * (DC_COLS + 1) + cl];             // (rows N .. NA - 1 of the state are zeros)
+                }
+#pragma unroll
+                for (int u = 0; u < DC_AHEAD; ++u)
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) acc[i] = fmaf(pv[u][i], cv[u], acc[i]);
             }
         }
         // the chunk begins with `run`; the next one with what has just been added up
 #pragma unroll
-        for (int i = 0; i < DC_MAX; ++i)
-            if (on && i < per && n0 + i < N) at[(size_t)(n0 + i) * vdim + col] = run[(n0 + i) * (DC_COLS + 1) + cl];
+        for (int i = 0; i < PER; ++i)
+            if (on && n0 + i < N) at[(size_t)(n0 + i) * vdim + col] = run[(n0 + i) * (DC_COLS + 1) + cl];
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < DC_MAX; ++i)
-            if (i < per && n0 + i < N) run[(n0 + i) * (DC_COLS + 1) + cl] = acc[i];
+        for (int i = 0; i < PER; ++i)
+            if (n0 + i < N) run[(n0 + i) * (DC_COLS + 1) + cl] = acc[i];
         __syncthreads();
     }
+}
+
+static void delta_carry_launch(float* carry, const float* pmat, const float* state, const int* slots, const int* q_len,
+                               const int* chunk_first, int heads, int vdim, int N, int Q, int segs, hipStream_t stream) {
+    const dim3 grid(segs, heads, (vdim + DC_COLS - 1) / DC_COLS);
+    const size_t lds = (size_t)((N + DC_ROUND - 1) / DC_ROUND * DC_ROUND) * (DC_COLS + 1) * sizeof(float);
+    const int per = (N + DC_SLICES - 1) / DC_SLICES;
+#define DC_GO(P_, V_) delta_carry_kernel<P_, 8, V_><<<grid, DC_COLS * DC_SLICES, lds, stream>>>(carry, pmat, state, slots, q_len, chunk_first, heads, vdim, N, Q)
+    const bool vec = N % 4 == 0 && ((uintptr_t)pmat % 16) == 0;
+    if (per <= 1) DC_GO(1, false); else if (per <= 2) DC_GO(2, false);
+    else if (per <= 4) { if (vec) DC_GO(4, true); else DC_GO(4, false); }
+    else if (per <= 8) { if (vec) DC_GO(8, true); else DC_GO(8, false); }
+    else { if (vec) DC_GO(16, true); else DC_GO(16, false); }
+#undef DC_GO
 }
 
 template <int NR, int NS, int CW>
@@ -820,8 +859,7 @@ static int delta_launch(const float* xkq, long x_stride, const float* ba, long b
     delta_scan_kernel<NR, NS, CW, 1><<<dim3(max_chunks, G * ub1), 64 * SSM_WAVES, lds, stream>>>(
         xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, pmat,
         y, y_stride, heads, vdim, N, G, Q, q_scale);
-    delta_carry_kernel<<<dim3(segs, heads, (vdim + DC_COLS - 1) / DC_COLS), DC_COLS * DC_SLICES,
-                         (size_t)N * (DC_COLS + 1) * sizeof(float), stream>>>(carry, pmat, state, slots, q_len, chunk_first, heads, vdim, N, Q);
+    delta_carry_launch(carry, pmat, state, slots, q_len, chunk_first, heads, vdim, N, Q, segs, stream);
     delta_scan_kernel<NR, NS, CW, 0><<<dim3(max_chunks, G * ub0), 64 * SSM_WAVES, lds, stream>>>(
         xkq, x_stride, ba, ba_stride, dt_bias, A_log, state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, pmat,
         y, y_stride, heads, vdim, N, G, Q, q_scale);
