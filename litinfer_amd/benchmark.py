@@ -795,8 +795,8 @@ def tovasun_latent_config(size: str, layers: int, vocab: int = 32000) -> Dict[st
 
 KUFOLORN_SIZES = {        # delta heads, their q/k heads; attention heads, kv heads; retention heads; key and value size of all three;
     # experts, identity outputs, chosen, groups, kept groups, expert width (four chosen experts are as wide as the dense feed-forward)
-    "1.5b": (12, 6, 12, 2, 4, 128, 12, 4, 4, 4, 3, 2240),
-    "7b": (28, 14, 28, 4, 8, 128, 12, 4, 4, 4, 3, 4736),
+    "1.5b": (12, 6, 12, 2, 4, 128, 14, 2, 4, 4, 2, 2240),
+    "7b": (28, 14, 28, 4, 8, 128, 14, 2, 4, 4, 2, 4736),
 }
 
 
@@ -810,10 +810,10 @@ def kufolorn_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, obj
            "router": {"experts": ne, "identity": ident, "top": top, "groups": {"count": groups, "keep": keep}}}
     delta = {"heads": dh, "kv_heads": dkv, "dim": dim, "vdim": dim, "conv": 4}
     par = {"left": {"heads": ah, "kv_heads": akv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
-                    "rot": {"base": 1000000.0, "dims": dim // 2, "scaling": {"factor": 2.0}}},
+                    "rot": {"base": 500000.0, "dims": dim // 2, "scaling": {"factor": 4.0}}},
            "right": {"heads": rh, "dim": dim, "vdim": dim, "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(rh)],
-                     "rot": {"base": 1000000.0, "dims": dim // 2}},
-           "left_scale": 0.6, "right_scale": 0.5}
+                     "rot": {"base": 500000.0, "dims": dim // 2}},
+           "left_scale": 0.7, "right_scale": 0.4}
     return {"architecture": "Kufolorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
             "layers": [{"type": "parallel" if i % 3 == 1 else "delta", "mixer": par if i % 3 == 1 else delta,
                         "mlp": dense if i % 2 == 0 else moe} for i in range(layers)]}

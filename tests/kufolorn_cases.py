@@ -57,11 +57,11 @@ CONFIG_B = {"architecture": "Kufolorn", "vocab": 300, "width": 128, "norm": {"ep
                        delta_layer(4, 1, 32, 32, 1, moe(4, 1, 1, 72, 2.0, 5, 5)),
                        delta_layer(3, 3, 16, 8, 5, dense(200))]}
 # C: sizes that reach the matrix-core kernels (head sizes 64 and 128, widths in multiples of 32), states of 128 and of 64
-# values a column, sixteen router outputs with identity experts that fill a whole group
-MOE_C = moe(12, 4, 3, 64, 2.0, 4, 3)
+# values a column, twelve router outputs in four groups of which two are kept, two of them identity experts
+MOE_C = moe(10, 2, 3, 64, 1.75, 4, 2)
 CONFIG_C = {"architecture": "Kufolorn", "vocab": 384, "width": 256, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
             "layers": [delta_layer(4, 2, 128, 64, 3, MOE_C),
-                       parallel_layer((8, 2, 64, 64, 0.125, rot(64, 1e6, 2.0)), (2, 64, 32, (0.98, 0.999), rot(64, 1e6)), 0.6, 0.5, dense(512)),
+                       parallel_layer((8, 2, 64, 64, 0.11, rot(64, 5e5, 3.0)), (2, 64, 64, (0.97, 0.9995), rot(32, 5e5)), 0.8, 0.3, dense(512)),
                        parallel_layer((4, 4, 128, 128, 0.09, rot(32, 1e4)), (4, 128, 64, (0.9, 0.95, 0.99, 0.999), rot(128)), 0.5, 0.5, MOE_C),
                        delta_layer(8, 8, 64, 32, 4, dense(256))]}
 # D: ones everywhere: one head, one q/k head, one expert chosen of one expert and one identity output, one group
